@@ -39,18 +39,7 @@
 #include "ktx_common.h"
 #include "ktx_internal.h"
 
-// =====================================================================================================
-// error slot
-// =====================================================================================================
-std::string& ktx_err_slot() {
-  static thread_local std::string s;
-  return s;
-}
-int ktx_fail(const std::string& msg) {
-  ktx_err_slot() = msg;
-  return -1;
-}
-extern "C" const char* ktx_last_error(void) { return ktx_err_slot().c_str(); }
+// (the error slot — ktx_fail / ktx_last_error — lives in ktx_err.hip, which the small sequence-mixer library links as well)
 
 // =====================================================================================================
 // device helpers

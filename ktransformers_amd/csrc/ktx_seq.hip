@@ -1,0 +1,678 @@
+// ktx_seq.hip — sequence-mixer kernels behind include/ktx_seq.h: sinusoidal embedding, a shape-agnostic dense GEMM (bf16 or
+// fp32 MFMA), sigmoid-weighted grouped-query attention with head mixing over a paged key cache (values = un-normed keys), the
+// mLSTM matrix-memory recurrence over state slots, and the fp32 RMS-norm glue that adds into the residual stream.
+//
+// Everything a recurrence or a score touches is fp32: the residual, norms, scores, attention weights and their mixing, gates,
+// exponentials and the state.  Element types only select how weights, activations and the key cache are stored and which MFMA
+// multiplies them.
+#include "ktx_common.h"
+#include "../../include/ktx_seq.h"
+
+#include <math.h>
+
+#include <algorithm>
+
+typedef __bf16 sq_v8bf __attribute__((ext_vector_type(8)));
+
+namespace {
+
+__device__ __forceinline__ float ld_elem(const float* p, size_t i) { return p[i]; }
+__device__ __forceinline__ float ld_elem(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }
+__device__ __forceinline__ void st_elem(float* p, size_t i, float v) { p[i] = v; }
+__device__ __forceinline__ void st_elem(bf16_t* p, size_t i, float v) { p[i] = (bf16_t)(ktx_pk_bf16(v, 0.f) & 0xffffu); }
+__device__ __forceinline__ bf16_t to_bf16_rne(float v) { return (bf16_t)(ktx_pk_bf16(v, 0.f) & 0xffffu); }
+
+// sum over the 256 threads of a workgroup; `red` = 4 floats of LDS; every thread gets the result
+__device__ __forceinline__ float block_sum256(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return ((red[0] + red[1]) + red[2]) + red[3];
+}
+
+__device__ __forceinline__ float sigmoid_f32(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float gelu_tanh_f32(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+__device__ __forceinline__ float log_sigmoid_f32(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+// ---------------------------------------------------------------------------------------------------------------------
+// embedding + sinusoidal positions
+template <typename WT>
+__global__ void __launch_bounds__(256) embed_sinpos_kernel(int width, int vocab, const int32_t* __restrict__ tok,
+                                                           const int32_t* __restrict__ pos, const WT* __restrict__ embed,
+                                                           const double* __restrict__ inv_freq, float* __restrict__ x) {
+  const int t = blockIdx.x;
+  int id = tok[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const double p = (double)pos[t];
+  for (int e = threadIdx.x; e < width; e += 256) {
+    const double ang = p * inv_freq[e >> 1];
+    const float s = (float)((e & 1) ? cos(ang) : sin(ang));
+    x[(size_t)t * width + e] = ld_elem(embed, (size_t)id * width + e) + s;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// dense GEMM  Y = act(A W^T): 64 x 64 tile, BK = 32, 4 wavefronts of 32 x 32; any shape (edges zero-filled / masked).
+template <typename T>
+struct GemmTraits;
+template <>
+struct GemmTraits<bf16_t> {
+  static constexpr int LDS_LD = 40;   // bf16 elements per tile row: 32 + 8 (16-byte aligned rows, 20-word stride)
+};
+template <>
+struct GemmTraits<float> {
+  static constexpr int LDS_LD = 33;   // odd word stride: the per-lane scalar fragment reads are conflict-free
+};
+
+template <typename AT, typename CT>
+__device__ __forceinline__ void gemm_stage(CT* dst, const AT* __restrict__ src, int64_t ld, int row0, int rows, int k0, int K,
+                                           bool vec) {
+  // thread -> (row = tid / 4, 8 consecutive k)
+  const int r = threadIdx.x >> 2, seg = (threadIdx.x & 3) * 8;
+  const int gr = row0 + r;
+  CT* d = dst + r * GemmTraits<CT>::LDS_LD + seg;
+  if (gr < rows && vec && k0 + seg + 8 <= K) {
+    const AT* s = src + (size_t)gr * ld + k0 + seg;
+    if constexpr (sizeof(AT) == 2 && sizeof(CT) == 2) {
+      *reinterpret_cast<uint4*>(d) = *reinterpret_cast<const uint4*>(s);
+    } else if constexpr (sizeof(AT) == 4 && sizeof(CT) == 2) {
+      const float4 a = *reinterpret_cast<const float4*>(s), b = *reinterpret_cast<const float4*>(s + 4);
+      uint4 o;
+      o.x = ktx_pk_bf16(a.x, a.y); o.y = ktx_pk_bf16(a.z, a.w); o.z = ktx_pk_bf16(b.x, b.y); o.w = ktx_pk_bf16(b.z, b.w);
+      *reinterpret_cast<uint4*>(d) = o;
+    } else {
+      const float4 a = *reinterpret_cast<const float4*>(s), b = *reinterpret_cast<const float4*>(s + 4);
+      d[0] = a.x; d[1] = a.y; d[2] = a.z; d[3] = a.w; d[4] = b.x; d[5] = b.y; d[6] = b.z; d[7] = b.w;
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int k = k0 + seg + i;
+    float v = 0.f;
+    if (gr < rows && k < K) v = ld_elem(src, (size_t)gr * ld + k);
+    if constexpr (sizeof(CT) == 2) d[i] = to_bf16_rne(v);
+    else d[i] = v;
+  }
+}
+
+template <typename AT, typename CT, typename YT>
+__global__ void __launch_bounds__(256) dense_gemm_kernel(int M, int N, int K, const AT* __restrict__ A, int64_t lda,
+                                                         const CT* __restrict__ W, YT* __restrict__ Y, int64_t ldy, int act,
+                                                         int ksplit, bool vec_a, bool vec_w) {
+  constexpr int LD = GemmTraits<CT>::LDS_LD;
+  __shared__ __attribute__((aligned(16))) CT As[64 * LD];
+  __shared__ __attribute__((aligned(16))) CT Ws[64 * LD];
+  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+  const int l16 = lane & 15, lq = lane >> 4;
+  v4f acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+  // K range of this workgroup (split-K over blockIdx.z in whole 32-wide steps)
+  const int ksteps = (K + 31) / 32;
+  const int per = (ksteps + ksplit - 1) / ksplit;
+  const int ks0 = blockIdx.z * per, ks1 = min(ksteps, ks0 + per);
+  for (int ks = ks0; ks < ks1; ks++) {
+    const int k0 = ks * 32;
+    __syncthreads();
+    gemm_stage<AT, CT>(As, A, lda, m0, M, k0, K, vec_a);
+    gemm_stage<CT, CT>(Ws, W, (int64_t)K, n0, N, k0, K, vec_w);
+    __syncthreads();
+    if constexpr (sizeof(CT) == 2) {
+      sq_v8bf af[2], bf[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        af[i] = *reinterpret_cast<const sq_v8bf*>(As + (wm + i * 16 + l16) * LD + lq * 8);
+        bf[i] = *reinterpret_cast<const sq_v8bf*>(Ws + (wn + i * 16 + l16) * LD + lq * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < 32; kk += 4) {
+        float af[2], bf[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+          af[i] = As[(wm + i * 16 + l16) * LD + kk + lq];
+          bf[i] = Ws[(wn + i * 16 + l16) * LD + kk + lq];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int m = m0 + wm + i * 16 + lq * 4 + r, n = n0 + wn + j * 16 + l16;
+        if (m < M && n < N) {
+          float v = acc[i][j][r];
+          if (ksplit > 1) {
+            if constexpr (sizeof(YT) == 4) atomicAdd(reinterpret_cast<float*>(Y) + (size_t)m * ldy + n, v);
+          } else {
+            if (act == KTX_ACT_GELU_TANH) v = gelu_tanh_f32(v);
+            st_elem(Y, (size_t)m * ldy + n, v);
+          }
+        }
+      }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// sigmoid attention: prep (q / k norms, temperature, cache append)
+template <typename KT>
+__global__ void __launch_bounds__(256) sigattn_prep_kernel(ktx_sigattn_config c, const float* __restrict__ proj, int64_t ldp,
+                                                           int q_off, int k_off, const float* __restrict__ wq,
+                                                           const float* __restrict__ wk, float eps, const int32_t* __restrict__ pos,
+                                                           const int32_t* __restrict__ loc, KT* __restrict__ kcache,
+                                                           float* __restrict__ kinv, float* __restrict__ q_out) {
+  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int H = c.heads, G = c.kv_heads, D = c.dim;
+  const float* row = proj + (size_t)t * ldp;
+  const int p = pos[t];
+  float temp = 1.f;
+  if (c.temp_coef != 0.f && c.temp_every > 0) temp = (float)(1.0 + (double)c.temp_coef * log((double)((p + 1) / c.temp_every) + 1.0));
+  const float qmul = temp * c.scale;
+  for (int u = wave; u < H + G; u += 4) {
+    const bool is_q = u < H;
+    const float* v = is_q ? row + q_off + (size_t)u * D : row + k_off + (size_t)(u - H) * D;
+    float ss = 0.f;
+    for (int d = lane; d < D; d += 64) ss += v[d] * v[d];
+    ss = wave_sum(ss);
+    const float rinv = 1.0f / sqrtf(ss / (float)D + eps);
+    if (is_q) {
+      float* o = q_out + ((size_t)t * H + u) * D;
+      for (int d = lane; d < D; d += 64) o[d] = v[d] * rinv * wq[d] * wk[d] * qmul;
+    } else {
+      const int g = u - H;
+      const size_t r = (size_t)loc[t];
+      KT* o = kcache + (r * G + g) * D;
+      for (int d = lane; d < D; d += 64) st_elem(o, d, v[d]);
+      if (lane == 0) kinv[r * G + g] = rinv;
+    }
+  }
+}
+
+// sigmoid attention, generic kernel: one query token x one key range per workgroup, fp32 on the vector ALUs.
+// LDS: qs [H*D] | ks [KC][kst] | ps [H][KC] | wm [H][KC] | kv [KC]   (floats; kst = G*D | 1)
+template <typename KT, typename OT, int NO>
+__global__ void __launch_bounds__(256) sigattn_fwd_kernel(ktx_sigattn_config c, int T, int KC, const float* __restrict__ q,
+                                                          const KT* __restrict__ kcache, const float* __restrict__ kinv,
+                                                          const int32_t* __restrict__ tok_req, const int32_t* __restrict__ pos,
+                                                          const int32_t* __restrict__ page_indptr,
+                                                          const int32_t* __restrict__ page_indices, const float* __restrict__ pb,
+                                                          const float* __restrict__ talk, float* __restrict__ partial,
+                                                          OT* __restrict__ out) {
+  extern __shared__ float lds[];
+  const int H = c.heads, G = c.kv_heads, D = c.dim, rep = H / G, GD = G * D, HD = H * D;
+  const int kst = GD | 1;
+  float* qs = lds;
+  float* ks = qs + HD;
+  float* ps = ks + (size_t)KC * kst;
+  float* wm = ps + H * KC;
+  const int t = blockIdx.x, split = blockIdx.y, nsplit = gridDim.y, tid = threadIdx.x;
+  const int p = pos[t], b = tok_req[t];
+  const int nkeys = p + 1;
+  int span = (nkeys + nsplit - 1) / nsplit;
+  span = (span + KC - 1) / KC * KC;
+  const int lo = split * span, hi = min(nkeys, lo + span);
+  const int32_t* pages = page_indices + page_indptr[b];
+  for (int e = tid; e < HD; e += 256) qs[e] = q[(size_t)t * HD + e];
+  float acc[NO];
+#pragma unroll
+  for (int i = 0; i < NO; i++) acc[i] = 0.f;
+  for (int j0 = lo; j0 < hi; j0 += KC) {
+    const int nk = min(KC, hi - j0);
+    __syncthreads();
+    // stage nk key rows (all key heads) as fp32
+    for (int e = tid; e < nk * GD; e += 256) {
+      const int jj = e / GD, x = e - jj * GD;
+      const int j = j0 + jj;
+      const size_t r = (size_t)pages[j / c.page_size] * c.page_size + (j % c.page_size);
+      ks[(size_t)jj * kst + x] = ld_elem(kcache, r * GD + x);
+    }
+    __syncthreads();
+    // scores -> weights
+    for (int e = tid; e < H * KC; e += 256) {
+      const int h = e / KC, jj = e - h * KC;
+      float w = 0.f;
+      if (jj < nk) {
+        const int g = h / rep, j = j0 + jj;
+        const float* qh = qs + h * D;
+        const float* kj = ks + (size_t)jj * kst + g * D;
+        float s = 0.f;
+        for (int d = 0; d < D; d++) s += qh[d] * kj[d];
+        const size_t r = (size_t)pages[j / c.page_size] * c.page_size + (j % c.page_size);
+        s *= kinv[r * G + g];
+        if (c.slope_span != 0.f) s -= exp2f(-c.slope_span * (float)(h + 1) / (float)H) * (float)(p - j);
+        w = sigmoid_f32(s + pb[h]);
+      }
+      ps[e] = w;
+    }
+    __syncthreads();
+    // head mixing
+    for (int e = tid; e < H * KC; e += 256) {
+      const int h = e / KC, jj = e - h * KC;
+      float w = 0.f;
+      for (int g = 0; g < H; g++) w += talk[h * H + g] * ps[g * KC + jj];
+      wm[e] = w;
+    }
+    __syncthreads();
+    // weights x values (values = the staged key rows)
+#pragma unroll
+    for (int i = 0; i < NO; i++) {
+      const int e = tid + i * 256;
+      if (e < HD) {
+        const int h = e / D, d = e - h * D, g = h / rep;
+        const float* wr = wm + h * KC;
+        const float* vc = ks + g * D + d;
+        float a = acc[i];
+        for (int jj = 0; jj < nk; jj++) a += wr[jj] * vc[(size_t)jj * kst];
+        acc[i] = a;
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NO; i++) {
+    const int e = tid + i * 256;
+    if (e < HD) {
+      if (nsplit > 1) partial[((size_t)split * T + t) * HD + e] = acc[i];
+      else st_elem(out, (size_t)t * HD + e, acc[i]);
+    }
+  }
+}
+
+template <typename OT>
+__global__ void __launch_bounds__(256) sigattn_reduce_kernel(int nsplit, size_t n, const float* __restrict__ partial,
+                                                             OT* __restrict__ out) {
+  const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= n) return;
+  float a = 0.f;
+  for (int s = 0; s < nsplit; s++) a += partial[(size_t)s * n + e];
+  st_elem(out, e, a);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// mLSTM recurrence: workgroup = (request, head, 64 value columns); wavefront w owns the rows d = w*DPG .. of the state slice,
+// lane = value column.  State slice, normaliser rows and the running maximum live in registers for the whole call.
+template <int DPG>
+__global__ void __launch_bounds__(256) mlstm_fwd_kernel(ktx_mlstm_config c, const int32_t* __restrict__ q_indptr,
+                                                        const int32_t* __restrict__ pos0, const int32_t* __restrict__ slot,
+                                                        const float* __restrict__ proj, int64_t ldp, int q_off, int k_off,
+                                                        int v_off, int i_off, int f_off, const float* __restrict__ ib,
+                                                        const float* __restrict__ fb, float* __restrict__ Sg,
+                                                        float* __restrict__ ng, float* __restrict__ mg,
+                                                        float* __restrict__ o_raw) {
+  extern __shared__ float lds[];
+  const int N = c.heads, D = c.dim, V = c.vdim;
+  float* qs = lds;              // [2][D]
+  float* kss = qs + 2 * D;      // [2][D]
+  float* red = kss + 2 * D;     // [4][64] partial outputs
+  float* redn = red + 256;      // [4]
+  const int b = blockIdx.x, hd = blockIdx.y, vs = blockIdx.z;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int v = vs * 64 + lane;
+  const bool vok = v < V;
+  const int t0 = q_indptr[b], t1 = q_indptr[b + 1];
+  if (t1 <= t0) return;
+  const int sl = slot[b];
+  const bool fresh = pos0[b] == 0;
+  const int d0 = wave * DPG;
+  float* Sp = Sg + ((size_t)sl * N + hd) * D * V;
+  float* np_ = ng + ((size_t)sl * N + hd) * D;
+  float S[DPG], nn[DPG];
+#pragma unroll
+  for (int i = 0; i < DPG; i++) {
+    const int d = d0 + i;
+    S[i] = (!fresh && d < D && vok) ? Sp[(size_t)d * V + v] : 0.f;
+    nn[i] = (!fresh && d < D) ? np_[d] : 0.f;
+  }
+  float m = fresh ? 0.f : mg[(size_t)sl * N + hd];
+  const float qscale = 1.0f / sqrtf((float)D);
+  const float bi = ib[hd], bf = fb[hd], cap = c.gate_cap;
+  for (int t = t0; t < t1; t++) {
+    const float* row = proj + (size_t)t * ldp;
+    const int buf = (t - t0) & 1;
+    float* qb = qs + buf * D;
+    float* kb = kss + buf * D;
+    for (int d = tid; d < D; d += 256) {
+      qb[d] = row[q_off + hd * D + d] * qscale;
+      kb[d] = row[k_off + hd * D + d];
+    }
+    const float vv = vok ? row[v_off + hd * V + v] : 0.f;
+    float zi = row[i_off + hd] + bi, zf = row[f_off + hd] + bf;
+    if (cap != 0.f) {
+      zi = cap * tanhf(zi / cap);
+      zf = cap * tanhf(zf / cap);
+    }
+    const float lf = log_sigmoid_f32(zf);
+    const float m_new = fmaxf(lf + m, zi);
+    const float a = expf(lf + m - m_new), bb = expf(zi - m_new);
+    m = m_new;
+    __syncthreads();
+    float po = 0.f, pn = 0.f;
+#pragma unroll
+    for (int i = 0; i < DPG; i++) {
+      const int d = d0 + i;
+      if (d < D) {
+        const float kd = kb[d], qd = qb[d];
+        const float bk = bb * kd;
+        S[i] = a * S[i] + bk * vv;
+        nn[i] = a * nn[i] + bk;
+        po += S[i] * qd;
+        pn += nn[i] * qd;
+      }
+    }
+    red[wave * 64 + lane] = po;
+    if (lane == 0) redn[wave] = pn;
+    __syncthreads();
+    if (wave == 0 && vok) {
+      const float num = ((red[lane] + red[64 + lane]) + red[128 + lane]) + red[192 + lane];
+      const float nq = ((redn[0] + redn[1]) + redn[2]) + redn[3];
+      const float den = fmaxf(fabsf(nq), expf(-m)) + c.denom_eps;
+      o_raw[(size_t)t * N * V + hd * V + v] = num / den;
+    }
+    // (the next token stages into the other q / k buffer; `red` is rewritten only behind the next token's first barrier)
+  }
+#pragma unroll
+  for (int i = 0; i < DPG; i++) {
+    const int d = d0 + i;
+    if (d < D) {
+      if (vok) Sp[(size_t)d * V + v] = S[i];
+      if (vs == 0 && lane == 0) np_[d] = nn[i];
+    }
+  }
+  if (vs == 0 && tid == 0) mg[(size_t)sl * N + hd] = m;
+}
+
+template <typename OT>
+__global__ void __launch_bounds__(256) mlstm_gate_norm_kernel(ktx_mlstm_config c, int T, const float* __restrict__ o_raw,
+                                                              const float* __restrict__ proj, int64_t ldp, int g_off,
+                                                              const float* __restrict__ w, OT* __restrict__ out) {
+  const int N = c.heads, V = c.vdim;
+  const int unit = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (unit >= T * N) return;
+  const int t = unit / N, hd = unit - t * N;
+  const float* o = o_raw + (size_t)t * N * V + hd * V;
+  float ss = 0.f;
+  for (int v = lane; v < V; v += 64) ss += o[v] * o[v];
+  ss = wave_sum(ss);
+  const float rinv = 1.0f / sqrtf(ss / (float)V + c.eps);
+  const float* g = proj + (size_t)t * ldp + g_off + hd * V;
+  for (int v = lane; v < V; v += 64) st_elem(out, (size_t)t * N * V + hd * V + v, o[v] * rinv * w[hd * V + v] * sigmoid_f32(g[v]));
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// fp32 norm glue (see the header); one workgroup per row, the row is re-read instead of staged
+template <typename OT>
+__global__ void __launch_bounds__(256) rms_combine_kernel(int W, const float* __restrict__ y1, const float* __restrict__ w1,
+                                                          const float* __restrict__ y2, const float* __restrict__ w2,
+                                                          const float* __restrict__ wn, int one_plus, float eps,
+                                                          float* __restrict__ xres, const int32_t* __restrict__ rows,
+                                                          OT* __restrict__ out) {
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const float* a = y1 + (size_t)(rows ? rows[t] : t) * W;
+  const float* b = y2 ? y2 + (size_t)t * W : nullptr;
+  float r1 = 1.f, r2 = 1.f;
+  if (b) {
+    float s1 = 0.f, s2 = 0.f;
+    for (int e = tid; e < W; e += 256) {
+      s1 += a[e] * a[e];
+      s2 += b[e] * b[e];
+    }
+    s1 = block_sum256(s1, red);
+    s2 = block_sum256(s2, red);
+    r1 = 1.0f / sqrtf(s1 / (float)W + eps);
+    r2 = 1.0f / sqrtf(s2 / (float)W + eps);
+  }
+  float rz = 1.f;
+  if (wn) {
+    float sz = 0.f;
+    for (int e = tid; e < W; e += 256) {
+      const float z = b ? 0.5f * (a[e] * r1 * w1[e] + b[e] * r2 * w2[e]) : a[e];
+      sz += z * z;
+    }
+    sz = block_sum256(sz, red);
+    rz = 1.0f / sqrtf(sz / (float)W + eps);
+  }
+  for (int e = tid; e < W; e += 256) {
+    const float z = b ? 0.5f * (a[e] * r1 * w1[e] + b[e] * r2 * w2[e]) : a[e];
+    const float r = wn ? z * rz * (one_plus ? 1.0f + wn[e] : wn[e]) : z;
+    if (xres) xres[(size_t)t * W + e] += r;
+    else st_elem(out, (size_t)t * W + e, r);
+  }
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+template <typename KT, typename OT>
+int sigattn_fwd_launch(const ktx_sigattn_config& c, int T, int KC, size_t lds, int nsplit, const float* q, const void* kc,
+                              const float* kinv, const int32_t* tr, const int32_t* pos, const int32_t* pip, const int32_t* pix,
+                              const float* pb, const float* talk, float* partial, void* out, hipStream_t st) {
+  const int HD = c.heads * c.dim;
+  const int no = (HD + 255) / 256;
+  const dim3 grid(T, nsplit);
+#define KTX_SA_GO(NO)                                                                                                      \
+  do {                                                                                                                     \
+    KTX_HIP(ktx_set_max_lds((const void*)sigattn_fwd_kernel<KT, OT, NO>, 160 * 1024));                                     \
+    sigattn_fwd_kernel<KT, OT, NO><<<grid, 256, lds, st>>>(c, T, KC, q, (const KT*)kc, kinv, tr, pos, pip, pix, pb, talk, partial, \
+                                                           (OT*)out);                                                      \
+  } while (0)
+  if (no <= 1) KTX_SA_GO(1);
+  else if (no <= 2) KTX_SA_GO(2);
+  else if (no <= 4) KTX_SA_GO(4);
+  else if (no <= 8) KTX_SA_GO(8);
+  else if (no <= 16) KTX_SA_GO(16);
+  else if (no <= 32) KTX_SA_GO(32);
+  else return ktx_fail("ktx_sigattn_forward: heads * dim must be <= 8192");
+#undef KTX_SA_GO
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+
+}  // namespace
+
+// =====================================================================================================================
+extern "C" {
+
+int ktx_embed_sinpos(int T, int width, int vocab, const int32_t* d_tokens, const int32_t* d_pos, const void* d_embed,
+                     int embed_dtype, const double* d_inv_freq, float* d_x, ktx_stream_t stream) {
+  KTX_REQUIRE(T >= 0 && width > 0 && vocab > 0, "ktx_embed_sinpos: T >= 0, width, vocab > 0");
+  KTX_REQUIRE(d_tokens && d_pos && d_embed && d_inv_freq && d_x, "ktx_embed_sinpos: null pointer");
+  if (T == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  if (embed_dtype == KTX_SEQ_BF16)
+    embed_sinpos_kernel<bf16_t><<<T, 256, 0, st>>>(width, vocab, d_tokens, d_pos, (const bf16_t*)d_embed, d_inv_freq, d_x);
+  else if (embed_dtype == KTX_SEQ_F32)
+    embed_sinpos_kernel<float><<<T, 256, 0, st>>>(width, vocab, d_tokens, d_pos, (const float*)d_embed, d_inv_freq, d_x);
+  else
+    return ktx_fail("ktx_embed_sinpos: unknown element type");
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_dense_gemm(int M, int N, int K, const void* d_A, int a_dtype, int64_t lda, const void* d_W, int w_dtype, void* d_Y,
+                   int y_dtype, int64_t ldy, int act, int ksplit, ktx_stream_t stream) {
+  KTX_REQUIRE(M >= 0 && N > 0 && K > 0, "ktx_dense_gemm: M >= 0, N, K > 0");
+  KTX_REQUIRE(d_A && d_W && d_Y, "ktx_dense_gemm: null pointer");
+  KTX_REQUIRE(lda >= K && ldy >= N, "ktx_dense_gemm: lda >= K and ldy >= N");
+  KTX_REQUIRE(act == KTX_ACT_NONE || act == KTX_ACT_GELU_TANH, "ktx_dense_gemm: unknown activation");
+  KTX_REQUIRE(ksplit >= 1 && (ksplit == 1 || (y_dtype == KTX_SEQ_F32 && act == KTX_ACT_NONE)),
+              "ktx_dense_gemm: split-K adds into a zeroed fp32 output and takes no activation");
+  KTX_REQUIRE(!(w_dtype == KTX_SEQ_F32 && a_dtype != KTX_SEQ_F32), "ktx_dense_gemm: an fp32 product needs fp32 activations");
+  if (M == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid((N + 63) / 64, (M + 63) / 64, ksplit);
+  KTX_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "ktx_dense_gemm: too many row tiles / splits");
+  const size_t asz = a_dtype == KTX_SEQ_F32 ? 4 : 2, wsz = w_dtype == KTX_SEQ_F32 ? 4 : 2;
+  const bool vec_a = aligned16(d_A) && (lda * asz) % 16 == 0 && K % 8 == 0;
+  const bool vec_w = aligned16(d_W) && ((size_t)K * wsz) % 16 == 0 && K % 8 == 0;
+#define KTX_GEMM_GO(AT, CT, YT)                                                                                          \
+  dense_gemm_kernel<AT, CT, YT><<<grid, 256, 0, st>>>(M, N, K, (const AT*)d_A, lda, (const CT*)d_W, (YT*)d_Y, ldy, act, ksplit, \
+                                                      vec_a, vec_w)
+  if (w_dtype == KTX_SEQ_BF16) {
+    if (a_dtype == KTX_SEQ_F32 && y_dtype == KTX_SEQ_F32) KTX_GEMM_GO(float, bf16_t, float);
+    else if (a_dtype == KTX_SEQ_F32 && y_dtype == KTX_SEQ_BF16) KTX_GEMM_GO(float, bf16_t, bf16_t);
+    else if (a_dtype == KTX_SEQ_BF16 && y_dtype == KTX_SEQ_F32) KTX_GEMM_GO(bf16_t, bf16_t, float);
+    else if (a_dtype == KTX_SEQ_BF16 && y_dtype == KTX_SEQ_BF16) KTX_GEMM_GO(bf16_t, bf16_t, bf16_t);
+    else return ktx_fail("ktx_dense_gemm: unknown element type");
+  } else if (w_dtype == KTX_SEQ_F32) {
+    if (y_dtype == KTX_SEQ_F32) KTX_GEMM_GO(float, float, float);
+    else return ktx_fail("ktx_dense_gemm: an fp32 product writes fp32");
+  } else {
+    return ktx_fail("ktx_dense_gemm: unknown element type");
+  }
+#undef KTX_GEMM_GO
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+static int sigattn_check(const ktx_sigattn_config* c, const char* who) {
+  if (!c || c->heads <= 0 || c->kv_heads <= 0 || c->dim <= 0 || c->heads % c->kv_heads != 0 || c->page_size <= 0 ||
+      (c->cache_dtype != KTX_SEQ_F32 && c->cache_dtype != KTX_SEQ_BF16))
+    return ktx_fail(std::string(who) + ": heads, kv_heads (dividing heads), dim, page_size must be positive and cache_dtype known");
+  return 0;
+}
+
+int ktx_sigattn_prep(const ktx_sigattn_config* cfg, int T, const float* d_proj, int64_t ldp, int q_off, int k_off,
+                     const float* d_wq, const float* d_wk, float eps, const int32_t* d_pos, const int32_t* d_cache_loc,
+                     void* d_kcache, float* d_kinv, float* d_q_out, ktx_stream_t stream) {
+  if (int rc = sigattn_check(cfg, "ktx_sigattn_prep")) return rc;
+  KTX_REQUIRE(T >= 0 && d_proj && d_wq && d_wk && d_pos && d_cache_loc && d_kcache && d_kinv && d_q_out, "ktx_sigattn_prep: null pointer");
+  KTX_REQUIRE(q_off >= 0 && k_off >= 0 && ldp >= (int64_t)q_off + cfg->heads * cfg->dim && ldp >= (int64_t)k_off + cfg->kv_heads * cfg->dim,
+              "ktx_sigattn_prep: q / k columns lie outside a row of proj");
+  if (T == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  if (cfg->cache_dtype == KTX_SEQ_BF16)
+    sigattn_prep_kernel<bf16_t><<<T, 256, 0, st>>>(*cfg, d_proj, ldp, q_off, k_off, d_wq, d_wk, eps, d_pos, d_cache_loc,
+                                                   (bf16_t*)d_kcache, d_kinv, d_q_out);
+  else
+    sigattn_prep_kernel<float><<<T, 256, 0, st>>>(*cfg, d_proj, ldp, q_off, k_off, d_wq, d_wk, eps, d_pos, d_cache_loc,
+                                                  (float*)d_kcache, d_kinv, d_q_out);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_sigattn_forward(const ktx_sigattn_config* cfg, int T, const float* d_q, const void* d_kcache, const float* d_kinv,
+                        const int32_t* d_tok_req, const int32_t* d_pos, const int32_t* d_page_indptr,
+                        const int32_t* d_page_indices, const float* d_pb, const float* d_talk, int nsplit, float* d_partial,
+                        void* d_out, int out_dtype, ktx_stream_t stream) {
+  if (int rc = sigattn_check(cfg, "ktx_sigattn_forward")) return rc;
+  KTX_REQUIRE(T >= 0 && d_q && d_kcache && d_kinv && d_tok_req && d_pos && d_page_indptr && d_page_indices && d_pb && d_talk && d_out,
+              "ktx_sigattn_forward: null pointer");
+  KTX_REQUIRE(nsplit >= 1 && nsplit <= 65535 && (nsplit == 1 || d_partial), "ktx_sigattn_forward: nsplit >= 1, with scratch when > 1");
+  KTX_REQUIRE(out_dtype == KTX_SEQ_F32 || out_dtype == KTX_SEQ_BF16, "ktx_sigattn_forward: unknown output type");
+  if (T == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  const ktx_sigattn_config& c = *cfg;
+  const size_t HD = (size_t)c.heads * c.dim, kst = ((size_t)c.kv_heads * c.dim) | 1;
+  // keys per staged chunk: the largest power of two (<= 64) whose rows fit 96 KiB of LDS beside q and the weight tiles
+  int KC = 64;
+  auto lds_of = [&](int kc) { return (HD + (size_t)kc * kst + 2 * (size_t)c.heads * kc + kc) * sizeof(float); };
+  while (KC > 1 && lds_of(KC) > 96 * 1024) KC >>= 1;
+  KTX_REQUIRE(lds_of(KC) <= 150 * 1024, "ktx_sigattn_forward: one key row of all heads does not fit the LDS");
+  const size_t lds = lds_of(KC);
+  int rc;
+  const bool direct = nsplit == 1;
+  if (c.cache_dtype == KTX_SEQ_BF16) {
+    if (direct && out_dtype == KTX_SEQ_BF16)
+      rc = sigattn_fwd_launch<bf16_t, bf16_t>(c, T, KC, lds, nsplit, d_q, d_kcache, d_kinv, d_tok_req, d_pos, d_page_indptr, d_page_indices, d_pb, d_talk, d_partial, d_out, st);
+    else
+      rc = sigattn_fwd_launch<bf16_t, float>(c, T, KC, lds, nsplit, d_q, d_kcache, d_kinv, d_tok_req, d_pos, d_page_indptr, d_page_indices, d_pb, d_talk, d_partial, d_out, st);
+  } else {
+    if (direct && out_dtype == KTX_SEQ_BF16)
+      rc = sigattn_fwd_launch<float, bf16_t>(c, T, KC, lds, nsplit, d_q, d_kcache, d_kinv, d_tok_req, d_pos, d_page_indptr, d_page_indices, d_pb, d_talk, d_partial, d_out, st);
+    else
+      rc = sigattn_fwd_launch<float, float>(c, T, KC, lds, nsplit, d_q, d_kcache, d_kinv, d_tok_req, d_pos, d_page_indptr, d_page_indices, d_pb, d_talk, d_partial, d_out, st);
+  }
+  if (rc) return rc;
+  if (!direct) {
+    const size_t n = (size_t)T * HD;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (out_dtype == KTX_SEQ_BF16) sigattn_reduce_kernel<bf16_t><<<blocks, 256, 0, st>>>(nsplit, n, d_partial, (bf16_t*)d_out);
+    else sigattn_reduce_kernel<float><<<blocks, 256, 0, st>>>(nsplit, n, d_partial, (float*)d_out);
+    KTX_HIP(hipGetLastError());
+  }
+  return 0;
+}
+
+int ktx_mlstm_forward(const ktx_mlstm_config* cfg, int B, const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_slot,
+                      const float* d_proj, int64_t ldp, int q_off, int k_off, int v_off, int i_off, int f_off, const float* d_ib,
+                      const float* d_fb, float* d_S, float* d_n, float* d_m, float* d_o_raw, ktx_stream_t stream) {
+  KTX_REQUIRE(cfg && cfg->heads > 0 && cfg->dim > 0 && cfg->vdim > 0, "ktx_mlstm_forward: heads, dim, vdim must be positive");
+  KTX_REQUIRE(cfg->dim <= 256, "ktx_mlstm_forward: dim must be <= 256 (a wavefront keeps dim / 4 state rows in registers)");
+  KTX_REQUIRE(B >= 0 && d_q_indptr && d_pos0 && d_slot && d_proj && d_ib && d_fb && d_S && d_n && d_m && d_o_raw,
+              "ktx_mlstm_forward: null pointer");
+  const int64_t need = std::max(std::max((int64_t)q_off + cfg->heads * cfg->dim, (int64_t)k_off + cfg->heads * cfg->dim),
+                                std::max((int64_t)v_off + cfg->heads * cfg->vdim, (int64_t)std::max(i_off, f_off) + cfg->heads));
+  KTX_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && i_off >= 0 && f_off >= 0 && ldp >= need,
+              "ktx_mlstm_forward: q / k / v / gate columns lie outside a row of proj");
+  if (B == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid(B, cfg->heads, (cfg->vdim + 63) / 64);
+  KTX_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "ktx_mlstm_forward: too many heads / value columns");
+  const size_t lds = (4 * (size_t)cfg->dim + 256 + 4) * sizeof(float);
+  const int dpg = (cfg->dim + 3) / 4;
+#define KTX_ML_GO(DPG)                                                                                                          \
+  mlstm_fwd_kernel<DPG><<<grid, 256, lds, st>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_proj, ldp, q_off, k_off, v_off, i_off, f_off, \
+                                                d_ib, d_fb, d_S, d_n, d_m, d_o_raw)
+  if (dpg <= 4) KTX_ML_GO(4);
+  else if (dpg <= 8) KTX_ML_GO(8);
+  else if (dpg <= 16) KTX_ML_GO(16);
+  else if (dpg <= 32) KTX_ML_GO(32);
+  else KTX_ML_GO(64);
+#undef KTX_ML_GO
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_mlstm_gate_norm(const ktx_mlstm_config* cfg, int T, const float* d_o_raw, const float* d_proj, int64_t ldp, int g_off,
+                        const float* d_w, void* d_out, int out_dtype, ktx_stream_t stream) {
+  KTX_REQUIRE(cfg && cfg->heads > 0 && cfg->vdim > 0, "ktx_mlstm_gate_norm: heads, vdim must be positive");
+  KTX_REQUIRE(T >= 0 && d_o_raw && d_proj && d_w && d_out, "ktx_mlstm_gate_norm: null pointer");
+  KTX_REQUIRE(g_off >= 0 && ldp >= (int64_t)g_off + cfg->heads * cfg->vdim, "ktx_mlstm_gate_norm: gate columns lie outside a row of proj");
+  if (T == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  const unsigned blocks = (unsigned)(((size_t)T * cfg->heads + 3) / 4);
+  if (out_dtype == KTX_SEQ_BF16) mlstm_gate_norm_kernel<bf16_t><<<blocks, 256, 0, st>>>(*cfg, T, d_o_raw, d_proj, ldp, g_off, d_w, (bf16_t*)d_out);
+  else if (out_dtype == KTX_SEQ_F32) mlstm_gate_norm_kernel<float><<<blocks, 256, 0, st>>>(*cfg, T, d_o_raw, d_proj, ldp, g_off, d_w, (float*)d_out);
+  else return ktx_fail("ktx_mlstm_gate_norm: unknown output type");
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_rms_combine(int T, int W, const float* d_y1, const float* d_w1, const float* d_y2, const float* d_w2, const float* d_wn,
+                    int one_plus, float eps, float* d_x_residual, const int32_t* d_rows, void* d_out, int out_dtype,
+                    ktx_stream_t stream) {
+  KTX_REQUIRE(T >= 0 && W > 0 && d_y1, "ktx_rms_combine: T >= 0, W > 0, y1 non-null");
+  KTX_REQUIRE(!d_y2 || (d_w1 && d_w2), "ktx_rms_combine: two inputs need their two weights");
+  KTX_REQUIRE(!d_y2 || !d_rows, "ktx_rms_combine: the row gather is for the single-input form");
+  KTX_REQUIRE((d_x_residual != nullptr) != (d_out != nullptr), "ktx_rms_combine: exactly one of x_residual / out");
+  if (T == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  if (d_x_residual || out_dtype == KTX_SEQ_F32)
+    rms_combine_kernel<float><<<T, 256, 0, st>>>(W, d_y1, d_w1, d_y2, d_w2, d_wn, one_plus, eps, d_x_residual, d_rows, (float*)d_out);
+  else if (out_dtype == KTX_SEQ_BF16)
+    rms_combine_kernel<bf16_t><<<T, 256, 0, st>>>(W, d_y1, d_w1, d_y2, d_w2, d_wn, one_plus, eps, d_x_residual, d_rows, (bf16_t*)d_out);
+  else
+    return ktx_fail("ktx_rms_combine: unknown output type");
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // extern "C"

@@ -152,3 +152,147 @@ class KDeepSeekV3Cache:
         page_idx = torch.where(ok, kv_indices[idx].to(local.dtype), torch.zeros_like(local))
         return page_idx, page_offset
 
+
+
+class ForwardBatch:
+    """What one scheduled step looks like to the sequence-mixer operators (include/ktx_seq.h): the tokens of all requests flattened,
+    int32 device tensors.  positions / tok_req / cache_loc per token; q_indptr / pos0 / slot / page_indptr per request;
+    page_indices = the requests' page lists back to back.  nsplit = workgroups that share one query token's keys."""
+    __slots__ = ("T", "B", "positions", "tok_req", "cache_loc", "q_indptr", "pos0", "slot", "page_indptr", "page_indices",
+                 "max_q_len", "max_kv_len", "nsplit")
+
+    def __init__(self, **kw):
+        for k in self.__slots__:
+            setattr(self, k, kw.get(k))
+
+
+class KHybridCache:
+    """Cache and state manager of decoders that mix paged attention with recurrent layers.
+
+    Per attention layer: one paged KEY cache [pages * page_size, kv_heads, dim] (bf16 or fp32) — the design's values are the
+    un-normed keys, so no value cache exists — and fp32 1 / rms(k) per row and key head; per recurrent layer: state slots
+    S [slots, heads, dim, vdim], n [slots, heads, dim], m [slots, heads] in fp32.  A request holds a list of pages (grown as it
+    grows) and one slot from admit() to release(); freed pages and slots go back on LIFO free lists and are handed out again
+    without being cleared: the attention kernels never read past a request's length and the recurrence starts from zero at
+    position 0 whatever the slot holds.
+
+    layer_specs: per layer {"attn": (kv_heads, dim) | None, "rec": (heads, dim, vdim) | None}.
+    plan() turns (request, n new tokens) pairs into a ForwardBatch; the operators append and read through it."""
+
+    def __init__(self, layer_specs, max_tokens: int, max_requests: int = 8, page_size: int = 64, dtype=torch.bfloat16,
+                 device="cuda:0"):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError("KHybridCache: bf16 or fp32 key cache")
+        self.layer_specs, self.page_size, self.dtype, self.device = list(layer_specs), int(page_size), dtype, torch.device(device)
+        self.max_requests = int(max_requests)
+        # every live request may leave one page partly filled
+        self.num_pages = (int(max_tokens) + self.page_size - 1) // self.page_size + self.max_requests
+        self.max_cache_len = self.num_pages * self.page_size
+        rows = self.num_pages * self.page_size
+        self.k_caches, self.k_inv, self.S, self.n, self.m = [], [], [], [], []
+        for spec in self.layer_specs:
+            a, r = spec.get("attn"), spec.get("rec")
+            self.k_caches.append(torch.zeros((rows, a[0], a[1]), dtype=dtype, device=self.device) if a else None)
+            self.k_inv.append(torch.zeros((rows, a[0]), dtype=torch.float32, device=self.device) if a else None)
+            self.S.append(torch.zeros((self.max_requests, r[0], r[1], r[2]), dtype=torch.float32, device=self.device) if r else None)
+            self.n.append(torch.zeros((self.max_requests, r[0], r[1]), dtype=torch.float32, device=self.device) if r else None)
+            self.m.append(torch.zeros((self.max_requests, r[0]), dtype=torch.float32, device=self.device) if r else None)
+        self.free_pages = list(range(self.num_pages - 1, -1, -1))
+        self.free_slots = list(range(self.max_requests - 1, -1, -1))
+        self.requests: Dict[Any, dict] = {}
+
+    # ---- allocation ------------------------------------------------------------------------------------------------
+    def admit(self, rid) -> None:
+        if rid in self.requests:
+            raise KeyError(f"KHybridCache: request {rid!r} is already live")
+        if not self.free_slots:
+            raise RuntimeError(f"KHybridCache: all {self.max_requests} state slots are in use")
+        self.requests[rid] = {"pages": [], "len": 0, "slot": self.free_slots.pop()}
+
+    def release(self, rid) -> None:
+        r = self.requests.pop(rid)
+        self.free_pages.extend(reversed(r["pages"]))
+        self.free_slots.append(r["slot"])
+
+    def seq_len(self, rid) -> int:
+        return self.requests[rid]["len"]
+
+    def live_tokens(self) -> int:
+        return sum(r["len"] for r in self.requests.values())
+
+    def _grow(self, r: dict, n_new: int) -> None:
+        need = (r["len"] + n_new + self.page_size - 1) // self.page_size - len(r["pages"])
+        if need > len(self.free_pages):
+            raise RuntimeError(f"KHybridCache: out of pages ({need} needed, {len(self.free_pages)} free of {self.num_pages})")
+        for _ in range(max(need, 0)):
+            r["pages"].append(self.free_pages.pop())
+
+    def plan(self, entries, target_workgroups: int = 1024, keys_per_split: int = 128) -> ForwardBatch:
+        """entries: [(request id, number of new tokens)], in batch order.  Grows each request's page list, advances its length and
+        returns the step's ForwardBatch (host lists -> device tensors, one copy each)."""
+        ps = self.page_size
+        positions, tok_req, cache_loc, q_indptr, pos0, slot, page_indptr, page_indices = [], [], [], [0], [], [], [0], []
+        max_q = max_kv = 0
+        for b, (rid, n_new) in enumerate(entries):
+            r = self.requests[rid]
+            self._grow(r, n_new)
+            start = r["len"]
+            pages = r["pages"]
+            for p in range(start, start + n_new):
+                positions.append(p)
+                tok_req.append(b)
+                cache_loc.append(pages[p // ps] * ps + p % ps)
+            r["len"] = start + n_new
+            q_indptr.append(q_indptr[-1] + n_new)
+            pos0.append(start)
+            slot.append(r["slot"])
+            page_indices.extend(pages)
+            page_indptr.append(len(page_indices))
+            max_q, max_kv = max(max_q, n_new), max(max_kv, r["len"])
+        T = len(positions)
+        dev = self.device
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+        nsplit = max(1, min(target_workgroups // max(T, 1), (max_kv + keys_per_split - 1) // keys_per_split))
+        return ForwardBatch(T=T, B=len(entries), positions=i32(positions), tok_req=i32(tok_req), cache_loc=i32(cache_loc),
+                            q_indptr=i32(q_indptr), pos0=i32(pos0), slot=i32(slot), page_indptr=i32(page_indptr),
+                            page_indices=i32(page_indices), max_q_len=max_q, max_kv_len=max_kv, nsplit=nsplit)
+
+    # ---- the single-request view util.generate.prefill_and_generate drives (one sequence, positions given by the caller) --------
+    SINGLE = "__single__"
+
+    def single_request_batch(self, position_ids: torch.Tensor) -> ForwardBatch:
+        """A ForwardBatch for ONE implicit request whose new tokens sit at `position_ids` ([T] or [1, T], consecutive).  All pages
+        the cache has are reserved for it at the first call, so a one-token step needs no host knowledge of the position: every
+        tensor is derived from position_ids on the device and a captured graph of the step stays valid as the sequence grows."""
+        ps = self.page_size
+        if self.SINGLE not in self.requests:
+            self.admit(self.SINGLE)
+            r = self.requests[self.SINGLE]
+            r["pages"] = [self.free_pages.pop() for _ in range(len(self.free_pages))]
+            r["page_t"] = torch.tensor(r["pages"], dtype=torch.int32, device=self.device)
+            r["slot_t"] = torch.tensor([r["slot"]], dtype=torch.int32, device=self.device)
+            r["page_indptr"] = torch.tensor([0, len(r["pages"])], dtype=torch.int32, device=self.device)
+            r["q_indptr1"] = torch.tensor([0, 1], dtype=torch.int32, device=self.device)
+            r["tok_req1"] = torch.zeros(1, dtype=torch.int32, device=self.device)
+        r = self.requests[self.SINGLE]
+        pos = position_ids.reshape(-1).to(device=self.device, dtype=torch.int32)
+        T = pos.numel()
+        loc = (r["page_t"][(pos // ps).long()] * ps + pos % ps).int()
+        cap = len(r["pages"]) * ps
+        one = T == 1     # (a one-token step allocates nothing on the host: it may be captured into a graph)
+        return ForwardBatch(T=T, B=1, positions=pos, cache_loc=loc, pos0=pos[:1],
+                            tok_req=r["tok_req1"] if one else torch.zeros(T, dtype=torch.int32, device=self.device),
+                            q_indptr=r["q_indptr1"] if one else torch.tensor([0, T], dtype=torch.int32, device=self.device),
+                            slot=r["slot_t"], page_indptr=r["page_indptr"], page_indices=r["page_t"], max_q_len=T, max_kv_len=cap,
+                            nsplit=max(1, min(1024, (cap + 127) // 128)) if one else 1)
+
+    def get_seq_length(self, layer_idx: Optional[int] = 0) -> int:
+        r = self.requests.get(self.SINGLE)
+        return r["len"] if r else 0
+
+    def get_max_length(self) -> Optional[int]:
+        return self.max_cache_len
+
+    def reset(self) -> None:
+        for rid in list(self.requests):
+            self.release(rid)

@@ -31,3 +31,30 @@ class RMSNorm(BaseInjectedModule):
 
 
 KQwen2MoeRMSNorm = KQwen3MoeRMSNorm = DeepseekV3RMSNorm = RMSNorm
+
+
+class KResidualRMSNorm(BaseInjectedModule):
+    """RMS norm of an fp32 residual stream: y / sqrt(mean(y^2) + eps) * w, or * (1 + w) for weights stored around zero (`one_plus`),
+    applied to a SUBLAYER'S OUTPUT and added into the residual in the same launch (post-norm decoders: x += norm(f(x))), or written
+    out in the compute type (the model's last norm, with an optional row gather so that only the wanted positions reach the head).
+    include/ktx_seq.h `ktx_rms_combine`.  The checkpoint tensor is the module's key itself (no `.weight` suffix) unless
+    `weight_suffix` says otherwise."""
+
+    def __init__(self, key: str, gguf_loader, config, orig_module, prefill_device: str = "cuda", generate_device: str = "cuda",
+                 one_plus: bool | None = None, weight_suffix: str = "", **kwargs):
+        BaseInjectedModule.__init__(self, key, gguf_loader, config, orig_module, prefill_device, generate_device, **kwargs)
+        object.__setattr__(self, "eps", float(orig_module.eps))
+        object.__setattr__(self, "one_plus", bool(orig_module.one_plus if one_plus is None else one_plus))
+        object.__setattr__(self, "weight_suffix", weight_suffix)
+        object.__setattr__(self, "weight_f32", None)
+
+    def load(self):
+        import torch
+        w = self.gguf_loader.load_tensor(self.key + self.weight_suffix, device=torch.device(self.device))
+        object.__setattr__(self, "weight_f32", w.to(torch.float32).contiguous())
+
+    def forward(self, y, residual=None, rows=None, out_dtype=None):
+        import torch
+        from ktransformers_amd._native_seq import rms_combine
+        return rms_combine(y, self.weight_f32, self.eps, one_plus=self.one_plus, residual=residual, rows=rows,
+                           out_dtype=out_dtype or torch.float32)

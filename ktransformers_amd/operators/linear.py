@@ -333,3 +333,23 @@ class KTransformersLinear(BaseInjectedModule):
             self.unload()
         else:
             raise ValueError("mode must be either InferenceState.GENERATE, InferenceState.PREFILL or InferenceState.UNLOAD")
+
+
+class KLinearDense(BaseInjectedModule):
+    """A bias-free linear of ANY shape in bf16 or fp32 (config.compute_dtype) whose checkpoint tensor is the module's key itself:
+    include/ktx_seq.h `ktx_dense_gemm` (bf16 or fp32 MFMA, fp32 accumulation, fp32 result).  The language-model head of the
+    fp32-residual decoders; KLinearTorch / KLinearMarlin keep serving the quantised families."""
+
+    def __init__(self, key: str, gguf_loader, config, orig_module: nn.Module, prefill_device: str = "cuda", generate_device: str = "cuda",
+                 weight_suffix: str = "", **kwargs):
+        BaseInjectedModule.__init__(self, key, gguf_loader, config, orig_module, prefill_device, generate_device, **kwargs)
+        object.__setattr__(self, "compute_dtype", getattr(config, "compute_dtype", torch.bfloat16))
+        object.__setattr__(self, "weight_suffix", weight_suffix)
+        object.__setattr__(self, "w", {})
+
+    def load(self):
+        self.w["w"] = self.gguf_loader.load_tensor(self.key + self.weight_suffix, device=torch.device(self.device)).to(self.compute_dtype).contiguous()
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        from ktransformers_amd._native_seq import dense_gemm
+        return dense_gemm(x.reshape(-1, x.shape[-1]), self.w["w"])

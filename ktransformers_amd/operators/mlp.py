@@ -99,3 +99,30 @@ class KDeepseekV3MLP(BaseInjectedModule):
 
 
 kDeepseekV3MLP = KDeepseekV3MLP
+
+
+class KDenseMLP(BaseInjectedModule):
+    """Two-matrix feed-forward W_down act(W_up h) on an fp32 residual stream (act = tanh-form GELU, applied in the epilogue of the up
+    GEMM: include/ktx_seq.h `ktx_dense_gemm`).  With the decoder layer's fusion hooks the post-norm and the residual add ride in
+    one `ktx_rms_combine` launch behind the down GEMM.  Checkpoint tensors: `<key>.up` [ff, width], `<key>.down` [width, ff]."""
+    SUPPORTS_FUSION = True
+
+    def __init__(self, key: str, gguf_loader, config, orig_module, prefill_device: str = "cuda", generate_device: str = "cuda",
+                 activation: str = "gelu_tanh", **kwargs):
+        BaseInjectedModule.__init__(self, key, gguf_loader, config, orig_module, prefill_device, generate_device, **kwargs)
+        object.__setattr__(self, "activation", activation)
+        object.__setattr__(self, "compute_dtype", getattr(config, "compute_dtype", torch.bfloat16))
+        object.__setattr__(self, "w", {})
+
+    def load(self):
+        dev = torch.device(self.device)
+        for n in ("up", "down"):
+            self.w[n] = self.gguf_loader.load_tensor(f"{self.key}.{n}", device=dev).to(self.compute_dtype).contiguous()
+
+    def forward(self, h, post_norm=None, residual=None):
+        from ktransformers_amd._native_seq import dense_gemm
+        a = dense_gemm(h, self.w["up"], out_dtype=self.compute_dtype, act=self.activation)
+        y = dense_gemm(a, self.w["down"])
+        if post_norm is not None and residual is not None:
+            return post_norm(y, residual=residual)
+        return y
