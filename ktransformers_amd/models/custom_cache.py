@@ -206,7 +206,7 @@ class KHybridCache:
         if rid in self.requests:
             raise KeyError(f"KHybridCache: request {rid!r} is already live")
         if not self.free_slots:
-            raise RuntimeError(f"KHybridCache: all {self.max_requests} state slots are in use")
+            self._add_slots(self.max_requests)
         self.requests[rid] = {"pages": [], "len": 0, "slot": self.free_slots.pop()}
 
     def release(self, rid) -> None:
@@ -223,9 +223,26 @@ class KHybridCache:
     def _grow(self, r: dict, n_new: int) -> None:
         need = (r["len"] + n_new + self.page_size - 1) // self.page_size - len(r["pages"])
         if need > len(self.free_pages):
-            raise RuntimeError(f"KHybridCache: out of pages ({need} needed, {len(self.free_pages)} free of {self.num_pages})")
+            self._add_pages(max(need - len(self.free_pages), self.num_pages // 2))
         for _ in range(max(need, 0)):
             r["pages"].append(self.free_pages.pop())
+
+    # The cache is sized by the caller's estimate (tokens and requests live at a time); a step that needs more gets it: the tensors are
+    # re-allocated with the old contents in front (new page / slot numbers follow the old ones), which invalidates captured graphs
+    # — the single-request view below reserves everything up front and never grows.
+    def _add_slots(self, extra: int) -> None:
+        grow = lambda t: None if t is None else torch.cat([t, torch.zeros((extra,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)])
+        self.S, self.n, self.m = [grow(t) for t in self.S], [grow(t) for t in self.n], [grow(t) for t in self.m]
+        self.free_slots.extend(range(self.max_requests + extra - 1, self.max_requests - 1, -1))
+        self.max_requests += extra
+
+    def _add_pages(self, extra: int) -> None:
+        rows = extra * self.page_size
+        grow = lambda t: None if t is None else torch.cat([t, torch.zeros((rows,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)])
+        self.k_caches, self.k_inv = [grow(t) for t in self.k_caches], [grow(t) for t in self.k_inv]
+        self.free_pages.extend(range(self.num_pages + extra - 1, self.num_pages - 1, -1))
+        self.num_pages += extra
+        self.max_cache_len = self.num_pages * self.page_size
 
     def plan(self, entries, target_workgroups: int = 1024, keys_per_split: int = 128) -> ForwardBatch:
         """entries: [(request id, number of new tokens)], in batch order.  Grows each request's page list, advances its length and

@@ -1,0 +1,374 @@
+"""Mitotar on the GPU against the plain CPU statement of the design (oracle/mitotar_ref.py, fp64): every mechanism alone through
+its kernel, then the model through the framework's registry, cache manager, step function and generation loops — whole prompts,
+token-by-token decoding, portions, unequal batches, reused pages and slots, keys far away and at page borders, odd sizes.
+Small random configurations; fp32 runs are held to rounding, bf16 runs to bf16 rounding."""
+import math
+
+import pytest
+import torch
+
+from oracle import mitotar_ref as R
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F32, BF16 = torch.float32, torch.bfloat16
+TOL = {F32: 3e-4, BF16: 6e-2}
+
+
+def rel(got, ref):
+    got, ref = got.detach().double().cpu(), ref.detach().double().cpu()
+    return float((got - ref).pow(2).mean().sqrt() / ref.pow(2).mean().sqrt().clamp_min(1e-30))
+
+
+def rows_rel(got, ref):
+    got, ref = got.detach().double().cpu(), ref.detach().double().cpu()
+    return float(((got - ref).pow(2).mean(-1).sqrt() / ref.pow(2).mean(-1).sqrt().clamp_min(1e-30)).max())
+
+
+def build(cfg, seed, dtype, max_tokens=2048, max_requests=8, page_size=16):
+    from ktransformers_amd.models import load_model
+    from ktransformers_amd.models.custom_cache import KHybridCache
+    from ktransformers_amd.models.modeling_mitotar import mitotar_layer_specs
+    from ktransformers_amd.util.loader import DictLoader
+    P = R.random_checkpoint(cfg, seed)
+    model, config, _ = load_model(cfg, dtype=dtype, device=DEV, loader=DictLoader(P))
+    cache = KHybridCache(mitotar_layer_specs(config), max_tokens, max_requests=max_requests, page_size=page_size, dtype=dtype, device=DEV)
+    return model, cache, P
+
+
+def tokens_of(cfg, n, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, cfg["vocab"], (n,), generator=g).tolist()
+
+
+def engine_of(model, cache):
+    from ktransformers_amd.util.batch_engine import BatchEngine
+    return BatchEngine(model, cache)
+
+
+CONFIGS = {
+    "gqa": dict(),                                                                              # heads 4 over 2 key heads
+    "odd": dict(width=40, vocab=53, heads=3, kv_heads=1, dim=12, r_heads=3, r_dim=5, r_vdim=7, ff=20, every=1, coef=0.7, eps=1e-3),
+    "wide_v": dict(width=48, heads=2, kv_heads=2, dim=40, r_heads=1, r_dim=24, r_vdim=80, n_layers=3, mlp_none_at=(1,), coef=0.0,
+                   gate_cap=3.0, scale=0.31),
+}
+
+
+# ---- mechanisms alone ----------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("width,vocab", [(64, 50), (37, 11)])
+def test_embedding_with_sinusoid_positions(dtype, width, vocab):
+    from ktransformers_amd._native_seq import embed_sinpos
+    g = torch.Generator().manual_seed(1)
+    table = torch.randn(vocab, width, generator=g).to(BF16)
+    tok = torch.randint(0, vocab, (9,), generator=g)
+    pos = torch.tensor([0, 1, 2, 63, 64, 1000, 4095, 77, 5])
+    inv = torch.pow(torch.tensor(10000.0, dtype=torch.float64), -2.0 * torch.arange((width + 1) // 2, dtype=torch.float64) / width)
+    got = embed_sinpos(tok.int().to(DEV), pos.int().to(DEV), table.to(dtype).to(DEV), inv.to(DEV))
+    ref = table.double()[tok] + R.sinusoid(pos, width)
+    assert (got.double().cpu() - ref).abs().max() < 1e-6
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("M,N,K", [(1, 5, 7), (3, 64, 32), (70, 130, 100), (65, 17, 264), (128, 192, 64)])
+def test_dense_gemm_any_shape(dtype, M, N, K):
+    from ktransformers_amd._native_seq import dense_gemm
+    g = torch.Generator().manual_seed(M * 1000 + N)
+    a = torch.randn(M, K, generator=g)
+    w = torch.randn(N, K, generator=g).to(BF16).float()
+    ref = (a.to(dtype).double() @ w.double().T)
+    got = dense_gemm(a.to(DEV), w.to(dtype).to(DEV))
+    assert rel(got, ref) < (1e-6 if dtype == F32 else 1e-6)      # the bf16 product of bf16-rounded operands is exact up to fp32 sums
+    got = dense_gemm(a.to(DEV), w.to(dtype).to(DEV), act="gelu_tanh", out_dtype=dtype)
+    assert rel(got, R.gelu_tanh(ref)) < (1e-5 if dtype == F32 else 6e-3)
+    got = dense_gemm(a.to(dtype).to(DEV), w.to(dtype).to(DEV), ksplit=3)
+    assert rel(got, ref) < 1e-6
+
+
+def test_norm_glue_forms():
+    from ktransformers_amd._native_seq import rms_combine
+    g = torch.Generator().manual_seed(3)
+    for W in (48, 37, 300):
+        y1, y2, x = (torch.randn(5, W, generator=g) for _ in range(3))
+        w1, w2, wn = (torch.randn(W, generator=g) for _ in range(3))
+        eps = 1e-3
+        z = 0.5 * (R.norm_plain(y1.double(), w1.double(), eps) + R.norm_plain(y2.double(), w2.double(), eps))
+        d = lambda t: t.to(DEV)
+        assert rel(rms_combine(d(y1), None, eps, y2=d(y2), w1=d(w1), w2=d(w2)), z) < 1e-6
+        xr = d(x.clone())
+        rms_combine(d(y1), d(wn), eps, one_plus=True, residual=xr, y2=d(y2), w1=d(w1), w2=d(w2))
+        assert rel(xr, x.double() + R.norm_one_plus(z, wn.double(), eps)) < 1e-6
+        xr = d(x.clone())
+        rms_combine(d(y1), d(wn), eps, one_plus=True, residual=xr)
+        assert rel(xr, x.double() + R.norm_one_plus(y1.double(), wn.double(), eps)) < 1e-6
+        rows = torch.tensor([4, 0, 0, 2], dtype=torch.int32)
+        got = rms_combine(d(y1), d(wn), eps, one_plus=False, rows=d(rows))
+        assert rel(got, R.norm_plain(y1.double(), wn.double(), eps)[rows.long()]) < 1e-6
+
+
+def _attn_case(seed, H, G, D, T, width=32, coef=0.5, every=4, scale=None, pb_mean=-1.0):
+    g = torch.Generator().manual_seed(seed)
+    c = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": scale or D ** -0.5, "q_temp": {"coef": coef, "every": every}}
+    P = {"a.q": torch.randn(H * D, width, generator=g) / math.sqrt(width), "a.k": torch.randn(G * D, width, generator=g) / math.sqrt(width),
+         "a.q.norm": 1 + 0.2 * torch.randn(D, generator=g), "a.k.norm": 1 + 0.2 * torch.randn(D, generator=g),
+         "a.talk": torch.eye(H) + 0.3 * torch.randn(H, H, generator=g), "a.pb": pb_mean + 0.5 * torch.randn(H, generator=g),
+         "a.o": torch.randn(width, H * D, generator=g) / math.sqrt(H * D)}
+    P = {k: v.to(BF16).double() for k, v in P.items()}
+    h = torch.randn(T, width, generator=g).to(BF16).double()
+    return c, P, h
+
+
+def _run_attention(c, P, h, dtype, chunks, page_size=8, nsplit=None, eps=1e-5):
+    """The operator's kernels on one request whose tokens arrive in `chunks`; returns the attention output before W_o."""
+    from ktransformers_amd._native_seq import dense_gemm, sigattn_config, sigattn_forward, sigattn_prep
+    from ktransformers_amd.models.custom_cache import KHybridCache
+    H, G, D = c["heads"], c["kv_heads"], c["dim"]
+    cache = KHybridCache([{"attn": (G, D), "rec": None}], 4096, max_requests=2, page_size=page_size, dtype=dtype, device=DEV)
+    cfg = sigattn_config(H, G, D, c["scale"], c["q_temp"]["coef"], c["q_temp"]["every"], 8.0, page_size, dtype)
+    w_in = torch.cat([P["a.q"], P["a.k"]]).to(dtype).to(DEV)
+    f = lambda n: P[n].float().to(DEV).contiguous()
+    cache.admit("r")
+    outs, at = [], 0
+    for n in chunks:
+        fb = cache.plan([("r", n)])
+        proj = dense_gemm(h[at:at + n].float().to(DEV), w_in)
+        q = sigattn_prep(cfg, proj, 0, H * D, f("a.q.norm"), f("a.k.norm"), eps, fb.positions, fb.cache_loc, cache.k_caches[0], cache.k_inv[0])
+        outs.append(sigattn_forward(cfg, q, cache.k_caches[0], cache.k_inv[0], fb.tok_req, fb.positions, fb.page_indptr, fb.page_indices,
+                                    f("a.pb"), f("a.talk"), nsplit=nsplit or fb.nsplit))
+        at += n
+    return torch.cat(outs)
+
+
+def _ref_attention(c, P, h, eps=1e-5):
+    P2 = dict(P)
+    P2["a.o"] = torch.eye(c["heads"] * c["dim"], dtype=torch.float64)
+    return R.sigmoid_talk_attention(P2, "a", c, h, eps)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("H,G,D", [(4, 2, 16), (3, 1, 12), (8, 8, 24), (2, 2, 5), (6, 3, 40)])
+def test_sigmoid_attention_whole_and_portions(dtype, H, G, D):
+    c, P, h = _attn_case(H * 100 + D, H, G, D, T=45)
+    ref = _ref_attention(c, P, h)
+    tol = TOL[dtype]
+    assert rel(_run_attention(c, P, h, dtype, [45]), ref) < tol
+    assert rel(_run_attention(c, P, h, dtype, [7, 2, 17, 1, 1, 16, 1]), ref) < tol          # portions, page borders inside them
+    assert rel(_run_attention(c, P, h, dtype, [40] + [1] * 5, nsplit=3), ref) < tol         # decoding with shared key ranges
+    assert rel(_run_attention(c, P, h, dtype, [45], page_size=64), ref) < tol
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("key_at", [0, 3, 7, 8, 15, 16, 63, 64, 333, 511, 512, 697, 698])
+def test_one_key_stands_out(dtype, key_at):
+    """A single (query, key) pair with a large score among ~700 keys whose weights are ~0: the output is that key's value row.  The
+    query is the last token, once as the end of a prompt and once decoded alone; keys at page borders, first tokens, far away."""
+    H, G, D, T = 2, 1, 64, 700
+    c, P, h = _attn_case(5, H, G, D, T, coef=0.0, pb_mean=-36.0, scale=1.0)
+    P["a.talk"] = torch.eye(H, dtype=torch.float64)
+    P["a.pb"] = torch.full((H,), -36.0, dtype=torch.float64)
+    # both query heads project like the key head and share its norm weight, and the key token's input is the query token's, three
+    # times as large (the norm takes the factor out of the score, the value row keeps it): q . k = dim for this pair and the pair
+    # of the query with itself, about +-sqrt(dim) for every other key, so with the bias at -36 only these two clear it
+    P["a.q"] = torch.cat([P["a.k"], P["a.k"]])
+    P["a.q.norm"] = P["a.k.norm"] = torch.ones(D, dtype=torch.float64)
+    h[key_at] = 3 * h[T - 1]
+    ref = _ref_attention(c, P, h)
+    for chunks in ([T], [T - 1, 1]):
+        got = _run_attention(c, P, h, dtype, chunks, page_size=8)
+        assert rel(got[-1], ref[-1]) < TOL[dtype], (key_at, chunks)
+    alone = _ref_attention(c, P, h[T - 1:])          # the query's pair with itself only
+    assert (ref[-1] - alone[0]).abs().max() > 1.0      # the far key does carry weight in the plain statement
+
+
+def _mlstm_case(seed, N, D, V, T, width=24, cap=6.0):
+    g = torch.Generator().manual_seed(seed)
+    c = {"heads": N, "dim": D, "vdim": V, "gate_cap": cap}
+    s = 1 / math.sqrt(width)
+    P = {"m.q": torch.randn(N * D, width, generator=g) * s, "m.k": torch.randn(N * D, width, generator=g) * s,
+         "m.v": torch.randn(N * V, width, generator=g) * s, "m.g": torch.randn(N * V, width, generator=g) * s,
+         "m.i": torch.randn(N, width, generator=g) * 2 * s, "m.f": torch.randn(N, width, generator=g) * 2 * s,
+         "m.i.b": torch.randn(N, generator=g), "m.f.b": 2 + torch.randn(N, generator=g), "m.norm": 1 + 0.2 * torch.randn(N * V, generator=g),
+         "m.o": torch.eye(N * V)}
+    P = {k: v.to(BF16).double() for k, v in P.items()}
+    return c, P, torch.randn(T, width, generator=g).to(BF16).double()
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("N,D,V", [(2, 8, 16), (1, 5, 7), (3, 48, 64), (1, 24, 80), (2, 130, 33)])
+def test_mlstm_whole_portions_and_state_carry(dtype, N, D, V):
+    from ktransformers_amd._native_seq import dense_gemm, mlstm_config, mlstm_forward, mlstm_gate_norm
+    from ktransformers_amd.models.custom_cache import KHybridCache
+    T, eps = 60, 1e-5
+    c, P, h = _mlstm_case(N * 50 + D, N, D, V, T)
+    ref = R.mlstm_mixer(P, "m", c, h, eps)
+    cfg = mlstm_config(N, D, V, c["gate_cap"], eps)
+    order = ("q", "k", "v", "g", "i", "f")
+    w_in = torch.cat([P["m." + n] for n in order]).to(dtype).to(DEV)
+    offs, at = {}, 0
+    for n in order:
+        offs[n] = at
+        at += P["m." + n].shape[0]
+    f = lambda n: P[n].float().to(DEV).contiguous()
+    for chunks in ([T], [1] * 6 + [2, 30, 3, 19]):
+        cache = KHybridCache([{"attn": None, "rec": (N, D, V)}], 256, max_requests=3, dtype=dtype, device=DEV)
+        cache.admit("x"), cache.admit("r")           # "r" sits in the second slot
+        cache.S[0].fill_(7.0), cache.n[0].fill_(-3.0), cache.m[0].fill_(5.0)       # a fresh request must not see what the slot held
+        outs, at = [], 0
+        for n in chunks:
+            fb = cache.plan([("r", n)])
+            proj = dense_gemm(h[at:at + n].float().to(DEV), w_in)
+            o = mlstm_forward(cfg, proj, offs, f("m.i.b"), f("m.f.b"), fb.q_indptr, fb.pos0, fb.slot, cache.S[0], cache.n[0], cache.m[0])
+            outs.append(mlstm_gate_norm(cfg, o, proj, offs["g"], f("m.norm"), F32))
+            at += n
+        assert rel(torch.cat(outs), ref) < TOL[dtype], chunks
+        assert float(cache.m[0][0].min()) == 5.0                                    # the other slot is untouched
+
+
+def test_mlstm_strong_gates_stay_finite():
+    """Large gate pre-activations (the cap binds), hundreds of steps: the running maximum keeps every exponential in range."""
+    from ktransformers_amd._native_seq import dense_gemm, mlstm_config, mlstm_forward
+    from ktransformers_amd.models.custom_cache import KHybridCache
+    N, D, V, T = 2, 8, 8, 400
+    c, P, h = _mlstm_case(9, N, D, V, T, cap=15.0)
+    P["m.i"] *= 40
+    P["m.f"] *= 40
+    q = (h @ P["m.q"].T).view(T, N, D) * D ** -0.5
+    i, f = R.mlstm_gates(P, "m", c, h)
+    ref, _ = R.mlstm_recurrence(q, (h @ P["m.k"].T).view(T, N, D), (h @ P["m.v"].T).view(T, N, V), i, f)
+    order = ("q", "k", "v", "g", "i", "f")
+    w_in = torch.cat([P["m." + n] for n in order]).float().to(DEV)
+    offs, at = {}, 0
+    for n in order:
+        offs[n] = at
+        at += P["m." + n].shape[0]
+    cache = KHybridCache([{"attn": None, "rec": (N, D, V)}], 512, max_requests=1, dtype=F32, device=DEV)
+    cache.admit("r")
+    fb = cache.plan([("r", T)])
+    o = mlstm_forward(mlstm_config(N, D, V, 15.0, 1e-5), dense_gemm(h.float().to(DEV), w_in), offs, P["m.i.b"].float().to(DEV),
+                      P["m.f.b"].float().to(DEV), fb.q_indptr, fb.pos0, fb.slot, cache.S[0], cache.n[0], cache.m[0])
+    assert torch.isfinite(o).all()
+    assert rel(o, ref.reshape(T, -1)) < 1e-3
+
+
+# ---- the model through registry, cache manager and step function ------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_whole_prompt_and_layers(dtype, name):
+    cfg = R.make_config(**CONFIGS[name])
+    model, cache, P = build(cfg, 11, dtype)
+    toks = tokens_of(cfg, 50, 1)
+    ref, ref_layers = R.forward(P, cfg, toks, return_layers=True)
+    cache.admit("a")
+    fb = cache.plan([("a", len(toks))])
+    logits, layers = model(torch.tensor(toks, dtype=torch.int32, device=DEV), None, cache, batch=fb, return_layers=True)
+    for li in range(len(cfg["layers"])):
+        assert rel(layers[li], ref_layers[li]) < TOL[dtype], f"layer {li}"
+    assert rows_rel(logits, ref) < (TOL[dtype] if dtype == F32 else 0.12)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("name", ["gqa", "odd"])
+def test_prefill_equals_token_by_token_and_portions(dtype, name):
+    cfg = R.make_config(**CONFIGS[name])
+    model, cache, P = build(cfg, 12, dtype, page_size=8)
+    eng = engine_of(model, cache)
+    toks = tokens_of(cfg, 41, 2)
+    ref = R.forward(P, cfg, toks)
+    want = list(range(len(toks)))
+    whole = eng.step([{"id": "w", "tokens": toks, "want": want}], ["w"])
+    tol = TOL[dtype] if dtype == F32 else 0.12
+    assert rows_rel(whole, ref) < tol
+    for sizes in ([1] * 41, [2] * 20 + [1], [3, 5, 8, 9, 16], [39, 2], [7] + [1] * 34):
+        got, at = [], 0
+        for k, n in enumerate(sizes):
+            got.append(eng.step([{"id": "p", "tokens": toks[at:at + n], "want": list(range(n))}], ["p"] if at + n == len(toks) else []))
+            at += n
+        got = torch.cat(got)
+        assert rows_rel(got, ref) < tol, sizes
+        # cutting the prompt differently changes the logits by rounding only
+        assert rows_rel(got, whole) < (2e-5 if dtype == F32 else 0.08), sizes
+    assert not cache.requests and len(cache.free_pages) == cache.num_pages
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_unequal_batch_equals_each_alone_and_reuses_pages_and_slots(dtype):
+    cfg = R.make_config(**CONFIGS["gqa"])
+    model, cache, P = build(cfg, 13, dtype, max_tokens=400, max_requests=3, page_size=8)
+    eng = engine_of(model, cache)
+    reqs = {"a": tokens_of(cfg, 1, 3), "b": tokens_of(cfg, 37, 4), "c": tokens_of(cfg, 90, 5)}
+    tail = 6
+    alone = {}
+    for rid, toks in reqs.items():
+        alone[rid] = R.forward(P, cfg, toks + tokens_of(cfg, tail, 50 + len(toks)))
+    tol = TOL[dtype] if dtype == F32 else 0.12
+    for round_ in range(3):       # every round takes the pages and slots the previous one gave back, in another order
+        order = list(reqs)[round_:] + list(reqs)[:round_]
+        lg = eng.step([{"id": r, "tokens": reqs[r], "want": [len(reqs[r]) - 1]} for r in order])
+        for k, r in enumerate(order):
+            assert rows_rel(lg[k:k + 1], alone[r][len(reqs[r]) - 1:len(reqs[r])]) < tol, (round_, r)
+        live = list(order)
+        for step in range(tail):
+            ext = {r: tokens_of(cfg, tail, 50 + len(reqs[r]))[step] for r in live}
+            ending = [r for r in live if (r == "a" and step == 1) or step == tail - 1]       # the short request leaves early
+            lg = eng.step([{"id": r, "tokens": [ext[r]], "want": [0]} for r in live], ending)
+            for k, r in enumerate(live):
+                p = len(reqs[r]) + step
+                assert rows_rel(lg[k:k + 1], alone[r][p:p + 1]) < tol, (round_, step, r)
+            live = [r for r in live if r not in ending]
+        assert not cache.requests
+
+
+@pytest.mark.parametrize("dtype", [F32])
+def test_long_decoding(dtype):
+    cfg = R.make_config(**CONFIGS["gqa"])
+    model, cache, P = build(cfg, 14, dtype, page_size=16)
+    eng = engine_of(model, cache)
+    toks = tokens_of(cfg, 330, 6)
+    ref = R.forward(P, cfg, toks)
+    got = [eng.step([{"id": "d", "tokens": toks[:10], "want": [9]}])]
+    for t in range(10, len(toks)):
+        got.append(eng.step([{"id": "d", "tokens": [toks[t]], "want": [0]}]))
+    assert rows_rel(torch.cat(got), ref[9:]) < TOL[dtype]
+
+
+def test_cache_grows_beyond_its_first_size():
+    cfg = R.make_config(**CONFIGS["gqa"])
+    model, cache, P = build(cfg, 15, F32, max_tokens=32, max_requests=1, page_size=8)
+    eng = engine_of(model, cache)
+    reqs = {k: tokens_of(cfg, 30 + 7 * k, k) for k in range(4)}          # more requests and tokens than the cache was made for
+    lg = eng.step([{"id": k, "tokens": t, "want": [len(t) - 1]} for k, t in reqs.items()])
+    for i, (k, t) in enumerate(reqs.items()):
+        assert rows_rel(lg[i:i + 1], R.forward(P, cfg, t)[-1:]) < TOL[F32]
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_greedy_generation_through_both_loops(dtype):
+    """util.generate.prefill_and_generate (one request, chunked prefill, the decode step replayed from a captured HIP graph) and
+    BatchEngine.generate (a batch of unequal prompts) against the plain statement's greedy continuation."""
+    from ktransformers_amd.models.custom_cache import KHybridCache
+    from ktransformers_amd.models.modeling_mitotar import mitotar_layer_specs
+    from ktransformers_amd.util.generate import prefill_and_generate
+    cfg = R.make_config(**CONFIGS["gqa"])
+    model, cache, P = build(cfg, 16, dtype, page_size=16)
+    prompts = {"p": tokens_of(cfg, 19, 7), "q": tokens_of(cfg, 5, 8)}
+    n_new = 12
+
+    def greedy_ref(toks):
+        """Teacher-forced on the framework's own tokens: every generated token must be the plain statement's argmax wherever its
+        margin is clear of rounding."""
+        return R.forward(P, cfg, toks)
+
+    out = engine_of(model, cache).generate(prompts, max_new_tokens=n_new)
+    for rid, prompt in prompts.items():
+        assert len(out[rid]) == n_new
+        lg = greedy_ref(prompt + out[rid])
+        for k, tok in enumerate(out[rid]):
+            row = lg[len(prompt) - 1 + k]
+            top2 = row.topk(2).values
+            if float(top2[0] - top2[1]) > (1e-3 if dtype == F32 else 0.25):
+                assert tok == int(row.argmax()), (rid, k)
+    for use_graph in (False, True):
+        c1 = KHybridCache(mitotar_layer_specs(model.config), 256, max_requests=1, page_size=16, dtype=dtype, device=DEV)
+        ids = torch.tensor([prompts["p"]], dtype=torch.int64, device=DEV)
+        toks = prefill_and_generate(model, ids, c1, max_new_tokens=n_new, use_cuda_graph=use_graph, chunk_size=8).tolist()
+        assert toks == out["p"], (use_graph, toks, out["p"])
