@@ -46,6 +46,9 @@ def _load() -> C.CDLL:
                                      C.c_float] + [C.c_void_p] * 6
     lib.ktx_sigattn_forward.argtypes = [C.POINTER(_SigAttnConfig), C.c_int] + [C.c_void_p] * 9 + [C.c_int, C.c_void_p, C.c_void_p, C.c_int,
                                                                                                  C.c_void_p]
+    lib.ktx_sigattn_prefill_eligible.argtypes = [C.POINTER(_SigAttnConfig)]
+    lib.ktx_sigattn_prefill.argtypes = [C.POINTER(_SigAttnConfig), C.c_int, C.c_int] + [C.c_void_p] * 11
+    lib.ktx_gelu_tanh.argtypes = [C.c_size_t, C.c_void_p, C.c_int, C.c_void_p]
     lib.ktx_mlstm_forward.argtypes = [C.POINTER(_MlstmConfig), C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64] + [
         C.c_int] * 5 + [C.c_void_p] * 7
     lib.ktx_mlstm_gate_norm.argtypes = [C.POINTER(_MlstmConfig), C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p,
@@ -99,6 +102,14 @@ def dense_gemm(a: torch.Tensor, w: torch.Tensor, out_dtype=torch.float32, act: s
         raise KtxError(f"dense_gemm: {a.dtype} {tuple(a.shape)} x {w.dtype} {tuple(w.shape)}^T does not fit")
     M, K = a.shape
     N = w.shape[0]
+    if (out is None and ksplit == 1 and M >= LIBRARY_GEMM_MIN_M and w.dtype == torch.bfloat16 and K % 64 == 0 and N % 8 == 0
+            and _library_gemm() is not None):
+        # prompt-sized bf16 products go to the library's tuned MFMA GEMM (include/ktx_gemm.h); the activation has its own launch
+        a16 = a if a.dtype == torch.bfloat16 else a.to(torch.bfloat16)
+        y = _library_gemm()(a16 if a16.stride(0) % 8 == 0 else a16.contiguous(), w, out_f32=out_dtype == torch.float32)
+        if ACT[act]:
+            check(lib.ktx_gelu_tanh(y.numel(), y.data_ptr(), SEQ_DTYPE[y.dtype], _stream_ptr(y.device)))
+        return y
     if out is None:
         out = (torch.zeros if ksplit > 1 else torch.empty)((M, N), dtype=out_dtype, device=a.device)
     elif out.dtype != out_dtype or tuple(out.shape) != (M, N) or out.stride(1) != 1:
@@ -106,6 +117,23 @@ def dense_gemm(a: torch.Tensor, w: torch.Tensor, out_dtype=torch.float32, act: s
     check(lib.ktx_dense_gemm(M, N, K, a.data_ptr(), SEQ_DTYPE[a.dtype], a.stride(0), w.data_ptr(), SEQ_DTYPE[w.dtype], out.data_ptr(),
                              SEQ_DTYPE[out_dtype], out.stride(0), ACT[act], int(ksplit), _stream_ptr(a.device)))
     return out
+
+
+LIBRARY_GEMM_MIN_M = 64
+_LIBRARY_GEMM: list = []
+
+
+def _library_gemm():
+    """ktransformers_amd._native.gemm_bf16_nt when the whole library is built, else None (libktx_seq.so alone: ktx_dense_gemm serves)."""
+    if not _LIBRARY_GEMM:
+        fn = None
+        if os.path.exists(LIB_PATHS[0]) and not os.environ.get("KTX_SEQ_OWN_GEMM"):
+            try:
+                from ktransformers_amd._native import gemm_bf16_nt as fn
+            except Exception:
+                fn = None
+        _LIBRARY_GEMM.append(fn)
+    return _LIBRARY_GEMM[0]
 
 
 def sigattn_config(heads: int, kv_heads: int, dim: int, scale: float, temp_coef: float, temp_every: int, slope_span: float,
@@ -143,6 +171,24 @@ def sigattn_forward(cfg: _SigAttnConfig, q: torch.Tensor, kcache: torch.Tensor, 
                                   page_indptr.data_ptr(), page_indices.data_ptr(), pb.data_ptr(), talk.data_ptr(), int(nsplit),
                                   partial.data_ptr() if partial is not None else None, out.data_ptr(), SEQ_DTYPE[out_dtype],
                                   _stream_ptr(q.device)))
+    return out
+
+
+def sigattn_prefill_eligible(cfg: _SigAttnConfig) -> bool:
+    return bool(lib.ktx_sigattn_prefill_eligible(C.byref(cfg)))
+
+
+def sigattn_prefill(cfg: _SigAttnConfig, q: torch.Tensor, kcache: torch.Tensor, kinv: torch.Tensor, q_indptr: torch.Tensor,
+                    pos0: torch.Tensor, page_indptr: torch.Tensor, page_indices: torch.Tensor, pb: torch.Tensor, talk: torch.Tensor,
+                    max_q_len: int) -> torch.Tensor:
+    """Prompt-sized calls on the matrix cores (ktx_sigattn_prefill) -> bf16 [T, heads * dim]."""
+    for t, what in ((q_indptr, "q_indptr"), (pos0, "pos0"), (page_indptr, "page_indptr"), (page_indices, "page_indices")):
+        _seq_dev(t, torch.int32, "sigattn_prefill " + what)
+    _seq_dev(q, torch.float32, "sigattn_prefill q")
+    out = torch.empty((q.shape[0], cfg.heads * cfg.dim), dtype=torch.bfloat16, device=q.device)
+    check(lib.ktx_sigattn_prefill(C.byref(cfg), pos0.numel(), int(max_q_len), q.data_ptr(), kcache.data_ptr(), kinv.data_ptr(),
+                                  q_indptr.data_ptr(), pos0.data_ptr(), page_indptr.data_ptr(), page_indices.data_ptr(), pb.data_ptr(),
+                                  talk.data_ptr(), out.data_ptr(), _stream_ptr(q.device)))
     return out
 
 

@@ -343,17 +343,38 @@ __global__ void __launch_bounds__(256) mlstm_fwd_kernel(ktx_mlstm_config c, cons
   float m = fresh ? 0.f : mg[(size_t)sl * N + hd];
   const float qscale = 1.0f / sqrtf((float)D);
   const float bi = ib[hd], bf = fb[hd], cap = c.gate_cap;
+  // the next token's inputs are requested a step ahead: their latency hides behind this token's update and barriers
+  float nq = 0.f, nk = 0.f, nv = 0.f, nzi = 0.f, nzf = 0.f;
+  {
+    const float* row = proj + (size_t)t0 * ldp;
+    if (tid < D) {
+      nq = row[q_off + hd * D + tid];
+      nk = row[k_off + hd * D + tid];
+    }
+    if (vok) nv = row[v_off + hd * V + v];
+    nzi = row[i_off + hd];
+    nzf = row[f_off + hd];
+  }
   for (int t = t0; t < t1; t++) {
-    const float* row = proj + (size_t)t * ldp;
     const int buf = (t - t0) & 1;
     float* qb = qs + buf * D;
     float* kb = kss + buf * D;
-    for (int d = tid; d < D; d += 256) {
-      qb[d] = row[q_off + hd * D + d] * qscale;
-      kb[d] = row[k_off + hd * D + d];
+    const float cq = nq, ck = nk, vv = nv;
+    float zi = nzi + bi, zf = nzf + bf;
+    if (t + 1 < t1) {
+      const float* row = proj + (size_t)(t + 1) * ldp;
+      if (tid < D) {
+        nq = row[q_off + hd * D + tid];
+        nk = row[k_off + hd * D + tid];
+      }
+      if (vok) nv = row[v_off + hd * V + v];
+      nzi = row[i_off + hd];
+      nzf = row[f_off + hd];
     }
-    const float vv = vok ? row[v_off + hd * V + v] : 0.f;
-    float zi = row[i_off + hd] + bi, zf = row[f_off + hd] + bf;
+    if (tid < D) {
+      qb[tid] = cq * qscale;
+      kb[tid] = ck;
+    }
     if (cap != 0.f) {
       zi = cap * tanhf(zi / cap);
       zf = cap * tanhf(zf / cap);
@@ -413,6 +434,259 @@ __global__ void __launch_bounds__(256) mlstm_gate_norm_kernel(ktx_mlstm_config c
   const float rinv = 1.0f / sqrtf(ss / (float)V + c.eps);
   const float* g = proj + (size_t)t * ldp + g_off + hd * V;
   for (int v = lane; v < V; v += 64) st_elem(out, (size_t)t * N * V + hd * V + v, o[v] * rinv * w[hd * V + v] * sigmoid_f32(g[v]));
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// decode-sized GEMM (M <= 8 rows): Y[m][n] = act(sum_k A[m][k] W[n][k]).  Bandwidth-bound on W: the activation rows sit in LDS in the
+// product's type, a wavefront owns RPW weight rows and streams them with 16-byte loads, fp32 accumulation, one wave reduction per row.
+template <typename AT, typename CT, typename YT, int MM>
+__global__ void __launch_bounds__(256) dense_gemv_kernel(int M, int N, int K, const AT* __restrict__ A, int64_t lda,
+                                                         const CT* __restrict__ W, YT* __restrict__ Y, int64_t ldy, int act, bool vec) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char gv_lds[];
+  CT* As = reinterpret_cast<CT*>(gv_lds);                 // [MM][Kp], Kp = K rounded up to 8
+  const int Kp = (K + 7) & ~7;
+  for (int e = threadIdx.x; e < MM * Kp; e += 256) {
+    const int m = e / Kp, k = e - m * Kp;
+    const float v = (m < M && k < K) ? ld_elem(A, (size_t)m * lda + k) : 0.f;
+    if constexpr (sizeof(CT) == 2) As[e] = to_bf16_rne(v);
+    else As[e] = v;
+  }
+  __syncthreads();
+  constexpr int RPW = 2;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+  for (int rr = 0; rr < RPW; rr++) {
+    const int n = (blockIdx.x * 4 + wave) * RPW + rr;
+    if (n >= N) break;
+    const CT* wrow = W + (size_t)n * K;
+    float acc[MM];
+#pragma unroll
+    for (int m = 0; m < MM; m++) acc[m] = 0.f;
+    for (int k = lane * 8; k < Kp; k += 512) {
+      float wv[8];
+      if (vec) {
+        if constexpr (sizeof(CT) == 2) {
+          const uint4 u = *reinterpret_cast<const uint4*>(wrow + k);
+          wv[0] = ktx_lo_f32(u.x); wv[1] = ktx_hi_f32(u.x); wv[2] = ktx_lo_f32(u.y); wv[3] = ktx_hi_f32(u.y);
+          wv[4] = ktx_lo_f32(u.z); wv[5] = ktx_hi_f32(u.z); wv[6] = ktx_lo_f32(u.w); wv[7] = ktx_hi_f32(u.w);
+        } else {
+          const float4 a = *reinterpret_cast<const float4*>(wrow + k), b = *reinterpret_cast<const float4*>(wrow + k + 4);
+          wv[0] = a.x; wv[1] = a.y; wv[2] = a.z; wv[3] = a.w; wv[4] = b.x; wv[5] = b.y; wv[6] = b.z; wv[7] = b.w;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) wv[i] = (k + i < K) ? ld_elem(wrow, (size_t)(k + i)) : 0.f;
+      }
+#pragma unroll
+      for (int m = 0; m < MM; m++) {
+        const CT* ar = As + m * Kp + k;
+        float a = acc[m];
+#pragma unroll
+        for (int i = 0; i < 8; i++) a = fmaf(wv[i], ld_elem(ar, (size_t)i), a);
+        acc[m] = a;
+      }
+    }
+#pragma unroll
+    for (int m = 0; m < MM; m++) {
+      float a = wave_sum(acc[m]);
+      if (lane == 0 && m < M) {
+        if (act == KTX_ACT_GELU_TANH) a = gelu_tanh_f32(a);
+        st_elem(Y, (size_t)m * ldy + n, a);
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) gelu_tanh_kernel(size_t n, T* __restrict__ y) {
+  const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (e < n) st_elem(y, e, gelu_tanh_f32(ld_elem(y, e)));
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// sigmoid attention, prompt-sized calls on the matrix cores.  Workgroup = 16 consecutive query rows of one request x ALL heads
+// (the head mixing needs every head's weight of a (query, key) pair in one place); wavefront w owns heads w, w + 4, ...
+// Per tile of 32 keys:  S_g = Q_g K^T (bf16 MFMA, Q fragments resident in registers) -> fp32 weights sigmoid(S kinv_j - slope (i - j)
+// + bias) into LDS -> every wavefront mixes its own heads' weights from all heads' (fp32 FMAs) -> bf16 -> O_h += W_h V (bf16 MFMA
+// against a transposed copy of the key tile: the values are the key rows).
+constexpr int SA_KN = 32;      // keys per tile
+constexpr int SA_PST = 33;     // row stride of the fp32 weight tiles (words)
+constexpr int SA_WST = 40;     // row stride of the bf16 mixed-weight / transposed-key tiles (elements)
+
+template <int NHW, int DS>
+__global__ void __launch_bounds__(256) sigattn_prefill_kernel(ktx_sigattn_config c, const float* __restrict__ q,
+                                                              const bf16_t* __restrict__ kcache, const float* __restrict__ kinv,
+                                                              const int32_t* __restrict__ q_indptr, const int32_t* __restrict__ pos0,
+                                                              const int32_t* __restrict__ page_indptr,
+                                                              const int32_t* __restrict__ page_indices, const float* __restrict__ pb,
+                                                              const float* __restrict__ talk, bf16_t* __restrict__ out) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char sa_lds[];
+  constexpr int D = DS * 32;
+  const int H = c.heads, G = c.kv_heads, rep = H / G, GD = G * D, HD = H * D;
+  const int KST = GD + 8;
+  bf16_t* ks = reinterpret_cast<bf16_t*>(sa_lds);                       // [32][KST]
+  bf16_t* vt = ks + SA_KN * KST;                                         // [GD][40]   transposed key tile
+  bf16_t* wm = vt + (size_t)GD * SA_WST;                                 // [H][16][40] mixed weights
+  float* ps = reinterpret_cast<float*>(wm + (size_t)H * 16 * SA_WST);    // [H][16][33] weights
+  float* kis = ps + (size_t)H * 16 * SA_PST;                             // [32][G]
+  float* tks = kis + SA_KN * G;                                          // [H][H]
+  const int b = blockIdx.y, tile = gridDim.x - 1 - blockIdx.x;            // long rows first
+  const int qb = q_indptr[b], qe = q_indptr[b + 1];
+  const int row0 = qb + tile * 16;
+  if (row0 >= qe) return;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
+  const int nrows = min(16, qe - row0);
+  const int p0 = pos0[b] + tile * 16;                 // position of row 0 of the tile
+  const int p_last = p0 + nrows - 1;
+  const int32_t* pages = page_indices + page_indptr[b];
+  for (int e = tid; e < H * H; e += 256) tks[e] = talk[e];
+  // Q fragments (A operand: row = l16, k = ds*32 + lq*8 ..)
+  sq_v8bf qf[NHW][DS];
+#pragma unroll
+  for (int u = 0; u < NHW; u++) {
+    const int g = wave + 4 * u;
+#pragma unroll
+    for (int ds = 0; ds < DS; ds++) {
+      uint4 pk = {0u, 0u, 0u, 0u};
+      if (g < H && l16 < nrows) {
+        const float* src = q + (size_t)(row0 + l16) * HD + g * D + ds * 32 + lq * 8;
+        const float4 a = *reinterpret_cast<const float4*>(src), bq = *reinterpret_cast<const float4*>(src + 4);
+        pk.x = ktx_pk_bf16(a.x, a.y); pk.y = ktx_pk_bf16(a.z, a.w); pk.z = ktx_pk_bf16(bq.x, bq.y); pk.w = ktx_pk_bf16(bq.z, bq.w);
+      }
+      qf[u][ds] = __builtin_bit_cast(sq_v8bf, pk);
+    }
+  }
+  v4f o[NHW][DS * 2];
+#pragma unroll
+  for (int u = 0; u < NHW; u++)
+#pragma unroll
+    for (int dn = 0; dn < DS * 2; dn++) o[u][dn] = (v4f){0.f, 0.f, 0.f, 0.f};
+  float slope[NHW], bias[NHW];
+#pragma unroll
+  for (int u = 0; u < NHW; u++) {
+    const int g = wave + 4 * u;
+    slope[u] = (g < H && c.slope_span != 0.f) ? exp2f(-c.slope_span * (float)(g + 1) / (float)H) : 0.f;
+    bias[u] = g < H ? pb[g] : 0.f;
+  }
+  const int chunks = GD / 8;                           // 16-byte pieces of one key row
+  for (int j0 = 0; j0 <= p_last; j0 += SA_KN) {
+    __syncthreads();
+    for (int e = tid; e < SA_KN * chunks; e += 256) {
+      const int jj = e / chunks, x = (e - jj * chunks) * 8;
+      const int j = j0 + jj;
+      uint4 v = {0u, 0u, 0u, 0u};
+      if (j <= p_last) {
+        const size_t r = (size_t)pages[j / c.page_size] * c.page_size + (j % c.page_size);
+        v = *reinterpret_cast<const uint4*>(kcache + r * GD + x);
+      }
+      *reinterpret_cast<uint4*>(ks + jj * KST + x) = v;
+      const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        vt[(size_t)(x + 2 * i) * SA_WST + jj] = (bf16_t)(w4[i] & 0xffffu);
+        vt[(size_t)(x + 2 * i + 1) * SA_WST + jj] = (bf16_t)(w4[i] >> 16);
+      }
+    }
+    for (int e = tid; e < SA_KN * G; e += 256) {
+      const int jj = e / G, g = e - jj * G, j = j0 + jj;
+      float v = 0.f;
+      if (j <= p_last) v = kinv[((size_t)pages[j / c.page_size] * c.page_size + (j % c.page_size)) * G + g];
+      kis[e] = v;
+    }
+    __syncthreads();
+    // scores -> weights (fp32) of this wavefront's heads
+#pragma unroll
+    for (int u = 0; u < NHW; u++) {
+      const int g = wave + 4 * u;
+      if (g < H) {
+        const int kg = g / rep;
+#pragma unroll
+        for (int nt = 0; nt < 2; nt++) {
+          v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ds = 0; ds < DS; ds++) {
+            const sq_v8bf kf = *reinterpret_cast<const sq_v8bf*>(ks + (nt * 16 + l16) * KST + kg * D + ds * 32 + lq * 8);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[u][ds], kf, acc, 0, 0, 0);
+          }
+          const int jj = nt * 16 + l16, j = j0 + jj;
+          const float ki = kis[jj * G + kg];
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            const int i = lq * 4 + r, pi = p0 + i;
+            float w = 0.f;
+            if (i < nrows && j <= pi) w = sigmoid_f32(acc[r] * ki - slope[u] * (float)(pi - j) + bias[u]);
+            ps[(g * 16 + i) * SA_PST + jj] = w;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    // head mixing (fp32), then bf16 for the value product
+    {
+      float wacc[NHW][8];
+#pragma unroll
+      for (int u = 0; u < NHW; u++)
+#pragma unroll
+        for (int x = 0; x < 8; x++) wacc[u][x] = 0.f;
+      for (int g = 0; g < H; g++) {
+        float pv[8];
+#pragma unroll
+        for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) pv[nt * 4 + r] = ps[(g * 16 + lq * 4 + r) * SA_PST + nt * 16 + l16];
+#pragma unroll
+        for (int u = 0; u < NHW; u++) {
+          const int h = wave + 4 * u;
+          const float tk = h < H ? tks[h * H + g] : 0.f;
+#pragma unroll
+          for (int x = 0; x < 8; x++) wacc[u][x] = fmaf(tk, pv[x], wacc[u][x]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < NHW; u++) {
+        const int h = wave + 4 * u;
+        if (h < H) {
+#pragma unroll
+          for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) wm[(h * 16 + lq * 4 + r) * SA_WST + nt * 16 + l16] = to_bf16_rne(wacc[u][nt * 4 + r]);
+        }
+      }
+    }
+    __syncthreads();
+    // O_h += W_h V
+#pragma unroll
+    for (int u = 0; u < NHW; u++) {
+      const int h = wave + 4 * u;
+      if (h < H) {
+        const int kg = h / rep;
+        const sq_v8bf wf = *reinterpret_cast<const sq_v8bf*>(wm + (h * 16 + l16) * SA_WST + lq * 8);
+#pragma unroll
+        for (int dn = 0; dn < DS * 2; dn++) {
+          const sq_v8bf vf = *reinterpret_cast<const sq_v8bf*>(vt + (size_t)(kg * D + dn * 16 + l16) * SA_WST + lq * 8);
+          o[u][dn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, vf, o[u][dn], 0, 0, 0);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < NHW; u++) {
+    const int h = wave + 4 * u;
+    if (h < H) {
+#pragma unroll
+      for (int dn = 0; dn < DS * 2; dn++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int i = lq * 4 + r;
+          if (i < nrows) out[(size_t)(row0 + i) * HD + h * D + dn * 16 + l16] = to_bf16_rne(o[u][dn][r]);
+        }
+    }
+  }
+}
+
+size_t sigattn_prefill_lds(const ktx_sigattn_config& c) {
+  const size_t GD = (size_t)c.kv_heads * c.dim, H = c.heads;
+  return SA_KN * (GD + 8) * 2 + GD * SA_WST * 2 + H * 16 * SA_WST * 2 + H * 16 * SA_PST * 4 + SA_KN * c.kv_heads * 4 + H * H * 4;
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -517,6 +791,35 @@ int ktx_dense_gemm(int M, int N, int K, const void* d_A, int a_dtype, int64_t ld
   KTX_REQUIRE(!(w_dtype == KTX_SEQ_F32 && a_dtype != KTX_SEQ_F32), "ktx_dense_gemm: an fp32 product needs fp32 activations");
   if (M == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
+  {
+    // decode-sized calls: the streaming kernel, when the activation rows fit the LDS
+    const size_t wsz0 = w_dtype == KTX_SEQ_F32 ? 4 : 2;
+    const int mm = M <= 2 ? 2 : 8;
+    const size_t lds = (size_t)mm * ((K + 7) & ~7) * wsz0;
+    if (M <= 8 && ksplit == 1 && lds <= 128 * 1024 && (w_dtype == KTX_SEQ_BF16 || y_dtype == KTX_SEQ_F32)) {
+      const bool vec = aligned16(d_W) && ((size_t)K * wsz0) % 16 == 0;
+      const unsigned blocks = (unsigned)((N + 7) / 8);
+#define KTX_GEMV_GO(AT, CT, YT, MM)                                                                                     \
+  do {                                                                                                                  \
+    KTX_HIP(ktx_set_max_lds((const void*)dense_gemv_kernel<AT, CT, YT, MM>, 128 * 1024));                               \
+    dense_gemv_kernel<AT, CT, YT, MM><<<blocks, 256, lds, st>>>(M, N, K, (const AT*)d_A, lda, (const CT*)d_W, (YT*)d_Y, ldy, act, vec); \
+  } while (0)
+#define KTX_GEMV_MM(AT, CT, YT)            \
+  do {                                     \
+    if (mm == 2) KTX_GEMV_GO(AT, CT, YT, 2); \
+    else KTX_GEMV_GO(AT, CT, YT, 8);       \
+  } while (0)
+      if (w_dtype == KTX_SEQ_F32) KTX_GEMV_MM(float, float, float);
+      else if (a_dtype == KTX_SEQ_F32 && y_dtype == KTX_SEQ_F32) KTX_GEMV_MM(float, bf16_t, float);
+      else if (a_dtype == KTX_SEQ_F32) KTX_GEMV_MM(float, bf16_t, bf16_t);
+      else if (y_dtype == KTX_SEQ_F32) KTX_GEMV_MM(bf16_t, bf16_t, float);
+      else KTX_GEMV_MM(bf16_t, bf16_t, bf16_t);
+#undef KTX_GEMV_MM
+#undef KTX_GEMV_GO
+      KTX_HIP(hipGetLastError());
+      return 0;
+    }
+  }
   const dim3 grid((N + 63) / 64, (M + 63) / 64, ksplit);
   KTX_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "ktx_dense_gemm: too many row tiles / splits");
   const size_t asz = a_dtype == KTX_SEQ_F32 ? 4 : 2, wsz = w_dtype == KTX_SEQ_F32 ? 4 : 2;
@@ -608,6 +911,59 @@ int ktx_sigattn_forward(const ktx_sigattn_config* cfg, int T, const float* d_q, 
     else sigattn_reduce_kernel<float><<<blocks, 256, 0, st>>>(nsplit, n, d_partial, (float*)d_out);
     KTX_HIP(hipGetLastError());
   }
+  return 0;
+}
+
+int ktx_sigattn_prefill_eligible(const ktx_sigattn_config* c) {
+  if (!c || sigattn_check(c, "ktx_sigattn_prefill_eligible")) return 0;
+  return c->cache_dtype == KTX_SEQ_BF16 && c->dim % 32 == 0 && c->dim <= 128 && c->heads <= 16 && sigattn_prefill_lds(*c) <= 150 * 1024;
+}
+
+int ktx_sigattn_prefill(const ktx_sigattn_config* cfg, int B, int max_q_len, const float* d_q, const void* d_kcache,
+                        const float* d_kinv, const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_page_indptr,
+                        const int32_t* d_page_indices, const float* d_pb, const float* d_talk, void* d_out, ktx_stream_t stream) {
+  KTX_REQUIRE(ktx_sigattn_prefill_eligible(cfg), "ktx_sigattn_prefill: needs a bf16 cache, dim % 32 == 0, dim <= 128, heads <= 16");
+  KTX_REQUIRE(B >= 0 && max_q_len >= 0 && d_q && d_kcache && d_kinv && d_q_indptr && d_pos0 && d_page_indptr && d_page_indices && d_pb &&
+                  d_talk && d_out, "ktx_sigattn_prefill: null pointer");
+  KTX_REQUIRE(B <= 65535, "ktx_sigattn_prefill: at most 65535 requests a call");
+  if (B == 0 || max_q_len == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  const ktx_sigattn_config& c = *cfg;
+  const dim3 grid((max_q_len + 15) / 16, B);
+  const size_t lds = sigattn_prefill_lds(c);
+  const int nhw = (c.heads + 3) / 4, ds = c.dim / 32;
+#define KTX_SP_GO(NHW, DS)                                                                                                   \
+  do {                                                                                                                       \
+    KTX_HIP(ktx_set_max_lds((const void*)sigattn_prefill_kernel<NHW, DS>, 160 * 1024));                                      \
+    sigattn_prefill_kernel<NHW, DS><<<grid, 256, lds, st>>>(c, d_q, (const bf16_t*)d_kcache, d_kinv, d_q_indptr, d_pos0,     \
+                                                            d_page_indptr, d_page_indices, d_pb, d_talk, (bf16_t*)d_out);    \
+  } while (0)
+#define KTX_SP_DS(NHW)                                                          \
+  do {                                                                          \
+    if (ds == 1) KTX_SP_GO(NHW, 1);                                             \
+    else if (ds == 2) KTX_SP_GO(NHW, 2);                                        \
+    else if (ds == 3) KTX_SP_GO(NHW, 3);                                        \
+    else KTX_SP_GO(NHW, 4);                                                     \
+  } while (0)
+  if (nhw <= 1) KTX_SP_DS(1);
+  else if (nhw <= 2) KTX_SP_DS(2);
+  else if (nhw <= 3) KTX_SP_DS(3);
+  else KTX_SP_DS(4);
+#undef KTX_SP_DS
+#undef KTX_SP_GO
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_gelu_tanh(size_t n, void* d_y, int dtype, ktx_stream_t stream) {
+  KTX_REQUIRE(d_y || n == 0, "ktx_gelu_tanh: null pointer");
+  if (n == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (dtype == KTX_SEQ_BF16) gelu_tanh_kernel<bf16_t><<<blocks, 256, 0, st>>>(n, (bf16_t*)d_y);
+  else if (dtype == KTX_SEQ_F32) gelu_tanh_kernel<float><<<blocks, 256, 0, st>>>(n, (float*)d_y);
+  else return ktx_fail("ktx_gelu_tanh: unknown element type");
+  KTX_HIP(hipGetLastError());
   return 0;
 }
 

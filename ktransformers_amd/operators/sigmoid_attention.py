@@ -20,6 +20,8 @@ from ktransformers_amd.operators.base_operator import BaseInjectedModule
 
 
 class KSigmoidTalkAttention(BaseInjectedModule):
+    PREFILL_MIN_Q = 16      # steps whose longest request brings at least this many tokens take the matrix-core kernel
+
     def __init__(self, key: str, gguf_loader, config, orig_module: nn.Module, prefill_device: str = "cuda", generate_device: str = "cuda",
                  **kwargs):
         BaseInjectedModule.__init__(self, key, gguf_loader, config, orig_module, prefill_device, generate_device, **kwargs)
@@ -57,13 +59,17 @@ class KSigmoidTalkAttention(BaseInjectedModule):
     def forward(self, h: torch.Tensor, batch, cache, proj: torch.Tensor | None = None, q_off: int = 0, k_off: int | None = None):
         """h: fp32 [T, width] (read only when `proj` is not given); proj: fp32 [T, *] holding W_q h at q_off and W_k h at k_off.
         Returns W_o(attention) as fp32 [T, width]."""
-        from ktransformers_amd._native_seq import dense_gemm, sigattn_forward, sigattn_prep
+        from ktransformers_amd._native_seq import dense_gemm, sigattn_forward, sigattn_prefill, sigattn_prefill_eligible, sigattn_prep
         if proj is None:
             proj = dense_gemm(h, torch.cat([self.w["q"], self.w["k"]]) if "qk" not in self.w else self.w["qk"])
             q_off, k_off = 0, self.heads * self.dim
         cfg = self._config(cache)
         kc, kinv = cache.k_caches[self.layer_idx], cache.k_inv[self.layer_idx]
         q = sigattn_prep(cfg, proj, q_off, k_off, self.w["q_norm"], self.w["k_norm"], self.eps, batch.positions, batch.cache_loc, kc, kinv)
+        if batch.max_q_len >= self.PREFILL_MIN_Q and self.compute_dtype == torch.bfloat16 and sigattn_prefill_eligible(cfg):
+            a = sigattn_prefill(cfg, q, kc, kinv, batch.q_indptr, batch.pos0, batch.page_indptr, batch.page_indices, self.w["pb"],
+                                self.w["talk"], batch.max_q_len)
+            return dense_gemm(a, self.w["o"])
         a = sigattn_forward(cfg, q, kc, kinv, batch.tok_req, batch.positions, batch.page_indptr, batch.page_indices, self.w["pb"],
                             self.w["talk"], nsplit=batch.nsplit, out_dtype=self.compute_dtype)
         return dense_gemm(a, self.w["o"])

@@ -49,6 +49,7 @@ def engine_of(model, cache):
 CONFIGS = {
     "gqa": dict(),                                                                              # heads 4 over 2 key heads
     "odd": dict(width=40, vocab=53, heads=3, kv_heads=1, dim=12, r_heads=3, r_dim=5, r_vdim=7, ff=20, every=1, coef=0.7, eps=1e-3),
+    "mfma": dict(width=128, vocab=200, heads=8, kv_heads=4, dim=32, r_heads=2, r_dim=32, r_vdim=64, ff=256, every=16),
     "wide_v": dict(width=48, heads=2, kv_heads=2, dim=40, r_heads=1, r_dim=24, r_vdim=80, n_layers=3, mlp_none_at=(1,), coef=0.0,
                    gate_cap=3.0, scale=0.31),
 }
@@ -155,6 +156,50 @@ def test_sigmoid_attention_whole_and_portions(dtype, H, G, D):
     assert rel(_run_attention(c, P, h, dtype, [7, 2, 17, 1, 1, 16, 1]), ref) < tol          # portions, page borders inside them
     assert rel(_run_attention(c, P, h, dtype, [40] + [1] * 5, nsplit=3), ref) < tol         # decoding with shared key ranges
     assert rel(_run_attention(c, P, h, dtype, [45], page_size=64), ref) < tol
+
+
+@pytest.mark.parametrize("H,G,D,T", [(4, 2, 32, 45), (8, 8, 96, 130), (6, 3, 64, 33), (16, 4, 128, 70), (1, 1, 32, 17), (13, 1, 64, 40)])
+def test_sigmoid_attention_matrix_core_kernel(H, G, D, T):
+    """The prompt kernel (16-row tiles x all heads, bf16 MFMA) against the plain statement: whole prompts, portions that start in the
+    middle of a tile and of a page, several requests of unequal length in one call."""
+    from ktransformers_amd._native_seq import dense_gemm, sigattn_config, sigattn_prefill, sigattn_prefill_eligible, sigattn_prep
+    from ktransformers_amd.models.custom_cache import KHybridCache
+    c, P, h = _attn_case(H * 7 + D, H, G, D, T)
+    ref = _ref_attention(c, P, h)
+    cfg = sigattn_config(H, G, D, c["scale"], c["q_temp"]["coef"], c["q_temp"]["every"], 8.0, 8, BF16)
+    assert sigattn_prefill_eligible(cfg)
+    w_in = torch.cat([P["a.q"], P["a.k"]]).to(BF16).to(DEV)
+    f = lambda n: P[n].float().to(DEV).contiguous()
+
+    def run(cache, plan, hs):
+        fb = cache.plan(plan)
+        proj = dense_gemm(torch.cat(hs).float().to(DEV), w_in)
+        q = sigattn_prep(cfg, proj, 0, H * D, f("a.q.norm"), f("a.k.norm"), 1e-5, fb.positions, fb.cache_loc, cache.k_caches[0], cache.k_inv[0])
+        return sigattn_prefill(cfg, q, cache.k_caches[0], cache.k_inv[0], fb.q_indptr, fb.pos0, fb.page_indptr, fb.page_indices,
+                               f("a.pb"), f("a.talk"), fb.max_q_len)
+
+    cache = KHybridCache([{"attn": (G, D), "rec": None}], 4096, max_requests=4, page_size=8, dtype=BF16, device=DEV)
+    cache.admit("r")
+    assert rel(run(cache, [("r", T)], [h]), ref) < TOL[BF16]
+    cache.admit("s"), cache.admit("t")
+    cut = T // 2 + 1
+    a = run(cache, [("s", cut), ("t", 3)], [h[:cut], h[:3]])            # two requests, then the rest of one as a second portion
+    assert rel(a[:cut], ref[:cut]) < TOL[BF16] and rel(a[cut:], ref[:3]) < TOL[BF16]
+    assert rel(run(cache, [("s", T - cut)], [h[cut:]]), ref[cut:]) < TOL[BF16]
+
+
+def test_prompt_sized_products_take_the_library_gemm():
+    from ktransformers_amd import _native_seq
+    g = torch.Generator().manual_seed(2)
+    a = torch.randn(200, 192, generator=g)
+    w = torch.randn(136, 192, generator=g).to(BF16)
+    ref = a.to(BF16).double() @ w.double().T
+    assert _native_seq._library_gemm() is not None
+    for out_dtype in (F32, BF16):
+        got = _native_seq.dense_gemm(a.to(DEV), w.to(DEV), out_dtype=out_dtype)
+        assert got.dtype == out_dtype and rel(got, ref) < (1e-6 if out_dtype == F32 else 4e-3)
+    got = _native_seq.dense_gemm(a.to(DEV), w.to(DEV), out_dtype=BF16, act="gelu_tanh")
+    assert rel(got, R.gelu_tanh(ref)) < 8e-3
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
