@@ -32,6 +32,7 @@ from __future__ import annotations
 import argparse
 import gc
 import json
+import math
 import os
 import shutil
 import subprocess
@@ -307,6 +308,8 @@ def rules_for(wl):
         name = r.get("match", {}).get("name", "")
         if kw.get("generate_op") == "KLinearMarlin" and name.startswith("^model\\.layers") and wl["linear"] == "FP8":
             kw["generate_op"] = "KLinearFP8"
+        if kw.get("generate_op") == "KLinearMarlin" and wl["linear"] == "BF16":
+            kw["generate_op"] = "KLinearTorch"
         if "backend" in kw:
             kw["backend"] = wl["experts"]
     fd, path = tempfile.mkstemp(prefix="ktx_rules_", suffix=".yaml", dir="/tmp")
@@ -1445,6 +1448,230 @@ def emit(out: dict) -> None:
     print(json.dumps(compact_line(out)), flush=True)
 
 
+# ---------------------------------------------------------------------------------------------------------------------
+# --mitotar: the fp32-residual sequence-mixer family (sigmoid head-mixing attention + mLSTM, models/modeling_mitotar.py) at a few
+# layer sizes, beside a dense DeepSeek-V2-Lite-geometry model (MLA + gated MLP, bf16 linears) of equal width / depth / parameters
+# ---------------------------------------------------------------------------------------------------------------------
+MITOTAR_SIZES = {
+    "w1024": dict(width=1024, heads=8, kv_heads=2, dim=128, r_heads=2, r_dim=128, r_vdim=512, ff=2816),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, dim=128, r_heads=4, r_dim=128, r_vdim=512, ff=5632),
+    "w4096": dict(width=4096, heads=16, kv_heads=4, dim=128, r_heads=8, r_dim=128, r_vdim=512, ff=11008),
+}
+MFMA_BF16_PEAK = 2.5e15
+
+
+class SeqRandomLoader:
+    """Random bf16 weights by tensor name for a Mitotar config (names and shapes of models/modeling_mitotar.py's checkpoint)."""
+
+    def __init__(self, cfg, dev):
+        self.dev, self.tensor_device_map, self.shapes = dev, {}, {}
+        W = cfg["width"]
+        self.shapes.update({"embed": (cfg["vocab"], W), "head": (cfg["vocab"], W), "final.norm": (W,)})
+        for i, L in enumerate(cfg["layers"]):
+            a, r, p = L["mixer"]["left"], L["mixer"]["right"], f"l{i}"
+            self.shapes.update({p + ".norm1": (W,), p + ".norm2": (W,), p + ".mix.left.q": (a["heads"] * a["dim"], W),
+                                p + ".mix.left.k": (a["kv_heads"] * a["dim"], W), p + ".mix.left.q.norm": (a["dim"],),
+                                p + ".mix.left.k.norm": (a["dim"],), p + ".mix.left.talk": (a["heads"], a["heads"]),
+                                p + ".mix.left.pb": (a["heads"],), p + ".mix.left.o": (W, a["heads"] * a["dim"]),
+                                p + ".mix.left.out": (W,), p + ".mix.right.out": (W,),
+                                p + ".mix.right.q": (r["heads"] * r["dim"], W), p + ".mix.right.k": (r["heads"] * r["dim"], W),
+                                p + ".mix.right.v": (r["heads"] * r["vdim"], W), p + ".mix.right.g": (r["heads"] * r["vdim"], W),
+                                p + ".mix.right.o": (W, r["heads"] * r["vdim"]), p + ".mix.right.norm": (r["heads"] * r["vdim"],),
+                                p + ".mix.right.i": (r["heads"], W), p + ".mix.right.f": (r["heads"], W),
+                                p + ".mix.right.i.b": (r["heads"],), p + ".mix.right.f.b": (r["heads"],),
+                                p + ".mlp.up": (L["mlp"]["ff"], W), p + ".mlp.down": (W, L["mlp"]["ff"])})
+
+    def has_tensor(self, name):
+        return name in self.shapes
+
+    def load_tensor(self, name, device="cpu"):
+        import zlib
+        shape = self.shapes[name]
+        g = torch.Generator(device=self.dev)
+        g.manual_seed(zlib.crc32(name.encode()))
+        t = torch.randn(shape, generator=g, device=self.dev, dtype=torch.bfloat16)
+        if name.endswith((".q.norm", ".k.norm", ".out", "right.norm")):
+            return t.mul_(0.1).add_(1.0)
+        if name.endswith(("norm1", "norm2", "final.norm")):
+            return t.mul_(0.1)
+        if name.endswith(".talk"):
+            return t.mul_(0.2 / shape[0] ** 0.5).add_(torch.eye(shape[0], device=self.dev, dtype=torch.bfloat16))
+        if name.endswith(".pb"):
+            return t.mul_(0.5).sub_(6.0)            # a few hundred keys carry weight, the rest next to none
+        if name.endswith(".f.b"):
+            return t.add_(3.0)
+        if len(shape) == 1 or name == "embed":
+            return t
+        return t.mul_(shape[-1] ** -0.5)
+
+
+class SeqKernelTimer:
+    """HIP events around every call of the sequence-mixer bindings (ktransformers_amd._native_seq) while active: the operators import
+    those functions at call time, so patching the module's attributes brackets each launch group.  Rows: name, calls, total ms,
+    algorithmic flops and bytes (from the call's shapes)."""
+    NAMES = ("embed_sinpos", "dense_gemm", "sigattn_prep", "sigattn_forward", "sigattn_prefill", "mlstm_forward", "mlstm_gate_norm",
+             "rms_combine")
+
+    def __init__(self, kv_len_of=None):
+        self.rows, self.saved, self.kv_len_of = [], {}, kv_len_of
+
+    def _cost(self, name, a, kw, out):
+        nb = lambda t: t.numel() * t.element_size() if isinstance(t, torch.Tensor) else 0
+        if name == "dense_gemm":
+            M, K = a[0].shape
+            N = a[1].shape[0]
+            return f"dense_gemm M={'prompt' if M > 8 else 'decode'}", 2.0 * M * N * K, nb(a[0]) + nb(a[1]) + nb(out)
+        if name in ("sigattn_forward", "sigattn_prefill"):
+            cfg, kc = a[0], a[2]
+            pairs, keys = self.kv_len_of()           # (query, key) pairs and cached keys read once, of the step at hand
+            gd = cfg.kv_heads * cfg.dim
+            return name, 4.0 * pairs * cfg.heads * cfg.dim, keys * (gd * kc.element_size() + 4 * cfg.kv_heads) + nb(a[1]) + nb(out)
+        if name == "mlstm_forward":
+            cfg, S = a[0], a[8]
+            B = a[7].numel()
+            return name, 0.0, 2.0 * B * cfg.heads * cfg.dim * cfg.vdim * 4 + nb(out)
+        return name, 0.0, sum(nb(t) for t in a) + nb(out)
+
+    def __enter__(self):
+        from ktransformers_amd import _native_seq
+        for name in self.NAMES:
+            fn = getattr(_native_seq, name)
+            self.saved[name] = fn
+
+            def wrapped(*a, _fn=fn, _name=name, **kw):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                out = _fn(*a, **kw)
+                e1.record()
+                self.rows.append((e0, e1) + self._cost(_name, a, kw, out))
+                return out
+            setattr(_native_seq, name, wrapped)
+        return self
+
+    def __exit__(self, *exc):
+        from ktransformers_amd import _native_seq
+        for name, fn in self.saved.items():
+            setattr(_native_seq, name, fn)
+
+    def table(self, total_ms):
+        torch.cuda.synchronize()
+        agg = {}
+        for e0, e1, label, flops, nbytes in self.rows:
+            a = agg.setdefault(label, [0, 0.0, 0.0, 0.0])
+            a[0] += 1
+            a[1] += e0.elapsed_time(e1)
+            a[2] += flops
+            a[3] += nbytes
+        out = []
+        for label, (n, ms, flops, nbytes) in sorted(agg.items(), key=lambda kv: -kv[1][1]):
+            t = ms * 1e-3
+            out.append({"kernel": label, "launches": n, "total_ms": round(ms, 3), "share": round(ms / total_ms, 4),
+                        "TFLOPs": round(flops / t / 1e12, 1) if flops else None, "GBs": round(nbytes / t / 1e9, 1),
+                        "frac_of_roof": round(max(flops / MFMA_BF16_PEAK, nbytes / (HBM_PEAK_GBS * 1e9)) / t, 4)})
+        return out
+
+
+def run_mitotar(args, dev):
+    """Prefill (one 2048-token prompt) and decode (batch 1 and 8 at a 2048-token context) throughput of Mitotar at MITOTAR_SIZES, each
+    beside a dense DeepSeek (MLA, V2-Lite geometry, bf16 linears) of equal width, depth and feed-forward parameters, with a per-kernel
+    table and the fraction of its roofline (bf16 MFMA peak or HBM peak, whichever bounds) for both.  Random weights, synthetic tokens.
+    Prints one JSON line; the whole record goes to bench_mitotar.json beside this file."""
+    import contextlib
+    import io
+    from ktransformers_amd.models import MODEL_REGISTRY, load_model
+    from ktransformers_amd.util.batch_engine import BatchEngine
+
+    n_layers, T, ctx = args.layers or 4, args.prefill_tokens, 2048
+    sizes = [s for s in (args.mitotar.split(",") if args.mitotar != "all" else MITOTAR_SIZES) if s in MITOTAR_SIZES]
+    record = {"metric": "mitotar_prefill_decode", "unit": "tok/s", "layers": n_layers, "prefill_tokens": T, "decode_ctx": ctx,
+              "dtype": "bf16 weights / activations / key cache, fp32 residual, scores, state", "data": "synthetic", "sizes": {}}
+
+    def timed_ms(fn, reps):
+        fn()
+        torch.cuda.synchronize(dev)
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize(dev)
+            ts.append((time.perf_counter() - t0) * 1e3)
+        return sorted(ts)[len(ts) // 2]
+
+    for name in sizes:
+        sz = MITOTAR_SIZES[name]
+        layer = {"type": "parallel", "mlp": {"kind": "dense", "ff": sz["ff"]},
+                 "mixer": {"left": {"heads": sz["heads"], "kv_heads": sz["kv_heads"], "dim": sz["dim"], "vdim": sz["dim"],
+                                    "scale": sz["dim"] ** -0.5, "q_temp": {"coef": 0.5, "every": 64}},
+                           "right": {"heads": sz["r_heads"], "dim": sz["r_dim"], "vdim": sz["r_vdim"], "gate_cap": 12.0}}}
+        cfg = {"architecture": "Mitotar", "width": sz["width"], "vocab": 32000, "norm": {"eps": 1e-6}, "layers": [layer] * n_layers}
+        with contextlib.redirect_stdout(io.StringIO()):
+            model, config, entry = load_model(cfg, dtype=torch.bfloat16, device=str(dev), loader=SeqRandomLoader(cfg, dev))
+        cache = entry.make_cache(config, 8 * (ctx + 64) + T, 16, torch.bfloat16, str(dev))
+        eng = BatchEngine(model, cache)
+        g = torch.Generator().manual_seed(5)
+        prompt = torch.randint(0, 32000, (T,), generator=g).tolist()
+        state = {"pairs": 0, "keys": 0}
+
+        def prefill():
+            state.update(pairs=T * (T + 1) // 2, keys=T)
+            eng.step([{"id": "p", "tokens": prompt, "want": [T - 1]}], ["p"])
+        ms = timed_ms(prefill, 3)
+        with SeqKernelTimer(lambda: (state["pairs"], state["keys"])) as kt:
+            prefill()
+        res = {"prefill": {"tok_s": round(T / ms * 1e3, 1), "ms": round(ms, 3), "per_kernel": kt.table(ms)}}
+        params = sum(math.prod(v) for k, v in SeqRandomLoader(cfg, dev).shapes.items() if k not in ("embed",))
+        for B in (1, 8):
+            ids = [f"d{b}" for b in range(B)]
+            ctx_prompt = torch.randint(0, 32000, (ctx,), generator=g).tolist()
+            eng.step([{"id": r, "tokens": ctx_prompt, "want": []} for r in ids])
+
+            def decode():
+                state.update(pairs=B * cache.seq_len(ids[0]), keys=B * cache.seq_len(ids[0]))
+                eng.step([{"id": r, "tokens": [7], "want": [0]} for r in ids])
+            ms = timed_ms(decode, 20)
+            with SeqKernelTimer(lambda: (state["pairs"], state["keys"])) as kt:
+                decode()
+            kv_bytes = n_layers * B * ctx * sz["kv_heads"] * sz["dim"] * 2
+            res[f"decode_bs{B}"] = {"tok_s": round(B / ms * 1e3, 1), "ms_per_step": round(ms, 3),
+                                    "frac_of_hbm_peak": round((params * 2 + kv_bytes) / (ms * 1e-3) / (HBM_PEAK_GBS * 1e9), 4),
+                                    "per_kernel": kt.table(ms), "graph": False}
+            for r in ids:
+                cache.release(r)
+        res["weights_GB"] = round(params * 2 / 1e9, 3)
+        del model, cache, eng
+        torch.cuda.empty_cache()
+        # ---- the closest existing family at equal size: DeepSeek skeleton, every layer dense, MLA of the V2-Lite geometry, bf16 linears
+        inter = int(round(sz["ff"] * 2 / 3 / 128)) * 128
+        MODELS["dense-" + name] = dict(MODELS["v2lite"], vocab_size=32000, hidden_size=sz["width"], intermediate_size=inter,
+                                       num_attention_heads=sz["width"] // 128, n_routed_experts=None, n_shared_experts=None,
+                                       first_k_dense_replace=n_layers)
+        wl = dict(model="dense-" + name, rules="DeepSeek-V2-Lite-Chat.yaml", linear="BF16", experts="AMXInt4", layers=n_layers,
+                  name="dense DeepSeek (MLA) " + name, H=sz["width"], I=inter, E=0, k=0, L=0, method="BF16", heads=sz["width"] // 128)
+        try:
+            mr = ModelDecodeRunner(wl, n_layers, dev, ctx, 64)
+            dms = timed(mr.step, 50, 10, dev, False) / 50 * 1e3
+            rows, _ = kernel_table(mr, dev, dms)
+            pf = whole_model_prefill(mr, T, dev)
+            res["deepseek_dense"] = {"intermediate": inter, "decode_bs1": {"tok_s": round(1e3 / dms, 1), "ms_per_step": round(dms, 3),
+                                                                          "graph": mr.graph_ok, "per_kernel": rows[:10]},
+                                     "prefill": {"tok_s": pf["value"], "ms": pf["ms_per_chunk"], "per_kernel": pf["per_kernel"]}}
+            del mr
+        except Exception as e:      # the comparison must not lose the new family's numbers
+            res["deepseek_dense"] = {"error": f"{type(e).__name__}: {e}"}
+        torch.cuda.empty_cache()
+        record["sizes"][name] = res
+        log(f"[mitotar] {name}: prefill {res['prefill']['tok_s']} tok/s, decode bs1 {res['decode_bs1']['tok_s']} tok/s, "
+            f"bs8 {res['decode_bs8']['tok_s']} tok/s")
+    with open(os.path.join(ROOT, "bench_mitotar.json"), "w") as f:
+        json.dump(record, f, indent=1)
+    line = {"metric": record["metric"], "unit": "tok/s", "layers": n_layers, "data": "synthetic",
+            "sizes": {k: {"prefill": v["prefill"]["tok_s"], "decode_bs1": v["decode_bs1"]["tok_s"], "decode_bs8": v["decode_bs8"]["tok_s"],
+                          "deepseek_dense_prefill": v["deepseek_dense"].get("prefill", {}).get("tok_s"),
+                          "deepseek_dense_decode_bs1": v["deepseek_dense"].get("decode_bs1", {}).get("tok_s")}
+                      for k, v in record["sizes"].items()}}
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -1480,6 +1707,10 @@ def main():
                     help="process-group backend of the N > 1 path.  nccl (= RCCL over xGMI) is the product path; gloo exists for the "
                          "one-GPU smoke of the N-process code path (ranks share cuda:0, the decode exchange still runs through the "
                          "peer-write transport over inter-process handles; RCCL refuses several ranks on one device)")
+    ap.add_argument("--mitotar", default="", metavar="SIZES",
+                    help="instead of the default workload: prefill / decode throughput of the Mitotar family (sigmoid head-mixing attention "
+                         "+ mLSTM mixers) at layer sizes from MITOTAR_SIZES (comma-separated, or 'all'), beside a dense DeepSeek of equal "
+                         "size; one JSON line, detail in bench_mitotar.json")
     ap.add_argument("--pmc-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--trace-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
@@ -1498,6 +1729,10 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a HIP device (no CPU fallback)"
     shared_gpu = dist_on and args.dist_backend == "gloo" and local_rank >= torch.cuda.device_count()
     dev = torch.device("cuda", local_rank % torch.cuda.device_count() if shared_gpu else local_rank)
+    if args.mitotar:
+        torch.cuda.set_device(dev)
+        run_mitotar(args, dev)
+        return
     torch.cuda.set_device(dev)
     if args.pmc_child:
         pmc_child(args, wl, dev)

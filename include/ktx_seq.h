@@ -65,14 +65,16 @@ int ktx_sigattn_forward(const ktx_sigattn_config* cfg, int T, const float* d_q, 
                         const int32_t* d_page_indices, const float* d_pb, const float* d_talk, int nsplit, float* d_partial,
                         void* d_out, int out_dtype, ktx_stream_t stream);
 
-/* Prompt-sized calls of the same operator on the matrix cores: request b's query rows q_indptr[b] .. q_indptr[b+1] (at most
- * max_q_len of them) start at position pos0[b]; workgroups of 16 query rows x all heads walk 32-key tiles: bf16 MFMA for Q K^T and
- * for weights x values (q rounded to bf16), scores / weights / head mixing in fp32.  out: bf16 [T][heads*dim].
+/* The same operator on the matrix cores, for prompts and for decode steps: request b's query rows q_indptr[b] .. q_indptr[b+1] (at
+ * most max_q_len of them; T rows in all) start at position pos0[b]; workgroups of 16 query rows x all heads walk 32-key tiles: bf16
+ * MFMA for Q K^T and for weights x values (q rounded to bf16), scores / weights / head mixing in fp32.  nsplit workgroups share a row
+ * tile's keys (partial sums in d_partial: fp32 [nsplit][T][heads*dim], then reduced).  out: bf16 [T][heads*dim].
  * Eligible: bf16 cache, dim % 32 == 0, dim <= 128, heads <= 16, tiles fit the LDS; ktx_sigattn_forward serves everything else. */
 int ktx_sigattn_prefill_eligible(const ktx_sigattn_config* cfg);
-int ktx_sigattn_prefill(const ktx_sigattn_config* cfg, int B, int max_q_len, const float* d_q, const void* d_kcache,
+int ktx_sigattn_prefill(const ktx_sigattn_config* cfg, int B, int T, int max_q_len, const float* d_q, const void* d_kcache,
                         const float* d_kinv, const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_page_indptr,
-                        const int32_t* d_page_indices, const float* d_pb, const float* d_talk, void* d_out, ktx_stream_t stream);
+                        const int32_t* d_page_indices, const float* d_pb, const float* d_talk, int nsplit, float* d_partial,
+                        void* d_out, ktx_stream_t stream);
 
 /* y = gelu_tanh(y) in place, n elements of `dtype` (the activation behind a GEMM that has no epilogue for it). */
 int ktx_gelu_tanh(size_t n, void* d_y, int dtype, ktx_stream_t stream);

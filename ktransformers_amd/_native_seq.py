@@ -47,7 +47,7 @@ def _load() -> C.CDLL:
     lib.ktx_sigattn_forward.argtypes = [C.POINTER(_SigAttnConfig), C.c_int] + [C.c_void_p] * 9 + [C.c_int, C.c_void_p, C.c_void_p, C.c_int,
                                                                                                  C.c_void_p]
     lib.ktx_sigattn_prefill_eligible.argtypes = [C.POINTER(_SigAttnConfig)]
-    lib.ktx_sigattn_prefill.argtypes = [C.POINTER(_SigAttnConfig), C.c_int, C.c_int] + [C.c_void_p] * 11
+    lib.ktx_sigattn_prefill.argtypes = [C.POINTER(_SigAttnConfig), C.c_int, C.c_int, C.c_int] + [C.c_void_p] * 9 + [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
     lib.ktx_gelu_tanh.argtypes = [C.c_size_t, C.c_void_p, C.c_int, C.c_void_p]
     lib.ktx_mlstm_forward.argtypes = [C.POINTER(_MlstmConfig), C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64] + [
         C.c_int] * 5 + [C.c_void_p] * 7
@@ -180,15 +180,18 @@ def sigattn_prefill_eligible(cfg: _SigAttnConfig) -> bool:
 
 def sigattn_prefill(cfg: _SigAttnConfig, q: torch.Tensor, kcache: torch.Tensor, kinv: torch.Tensor, q_indptr: torch.Tensor,
                     pos0: torch.Tensor, page_indptr: torch.Tensor, page_indices: torch.Tensor, pb: torch.Tensor, talk: torch.Tensor,
-                    max_q_len: int) -> torch.Tensor:
-    """Prompt-sized calls on the matrix cores (ktx_sigattn_prefill) -> bf16 [T, heads * dim]."""
+                    max_q_len: int, nsplit: int = 1) -> torch.Tensor:
+    """The matrix-core kernel, prompts and decode steps (ktx_sigattn_prefill) -> bf16 [T, heads * dim]."""
     for t, what in ((q_indptr, "q_indptr"), (pos0, "pos0"), (page_indptr, "page_indptr"), (page_indices, "page_indices")):
         _seq_dev(t, torch.int32, "sigattn_prefill " + what)
     _seq_dev(q, torch.float32, "sigattn_prefill q")
-    out = torch.empty((q.shape[0], cfg.heads * cfg.dim), dtype=torch.bfloat16, device=q.device)
-    check(lib.ktx_sigattn_prefill(C.byref(cfg), pos0.numel(), int(max_q_len), q.data_ptr(), kcache.data_ptr(), kinv.data_ptr(),
+    T, HD = q.shape[0], cfg.heads * cfg.dim
+    out = torch.empty((T, HD), dtype=torch.bfloat16, device=q.device)
+    partial = torch.empty((nsplit, T, HD), dtype=torch.float32, device=q.device) if nsplit > 1 else None
+    check(lib.ktx_sigattn_prefill(C.byref(cfg), pos0.numel(), T, int(max_q_len), q.data_ptr(), kcache.data_ptr(), kinv.data_ptr(),
                                   q_indptr.data_ptr(), pos0.data_ptr(), page_indptr.data_ptr(), page_indices.data_ptr(), pb.data_ptr(),
-                                  talk.data_ptr(), out.data_ptr(), _stream_ptr(q.device)))
+                                  talk.data_ptr(), int(nsplit), partial.data_ptr() if partial is not None else None, out.data_ptr(),
+                                  _stream_ptr(q.device)))
     return out
 
 

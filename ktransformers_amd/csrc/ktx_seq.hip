@@ -504,33 +504,36 @@ __global__ void __launch_bounds__(256) gelu_tanh_kernel(size_t n, T* __restrict_
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
-// sigmoid attention, prompt-sized calls on the matrix cores.  Workgroup = 16 consecutive query rows of one request x ALL heads
-// (the head mixing needs every head's weight of a (query, key) pair in one place); wavefront w owns heads w, w + 4, ...
+// sigmoid attention on the matrix cores (prompts AND decode steps).  Workgroup = 16 consecutive query rows of one request x ALL
+// heads (the head mixing needs every head's weight of a (query, key) pair in one place) x one range of the keys; wavefront w owns the
+// NHW consecutive heads w*NHW .. (with grouped queries they share their key head, so its fragments are loaded once).
 // Per tile of 32 keys:  S_g = Q_g K^T (bf16 MFMA, Q fragments resident in registers) -> fp32 weights sigmoid(S kinv_j - slope (i - j)
-// + bias) into LDS -> every wavefront mixes its own heads' weights from all heads' (fp32 FMAs) -> bf16 -> O_h += W_h V (bf16 MFMA
-// against a transposed copy of the key tile: the values are the key rows).
+// + bias) into LDS -> every wavefront mixes its own heads' weights from all heads' (fp32 FMAs) -> bf16 -> O_h += W_h V (bf16 MFMA; the
+// values are the key rows, read from the same LDS tile column-wise).  Weights are not normalised over keys, so the key ranges of a
+// row (gridDim.z of them) are plain partial sums: fp32 partials + ktx's reduce kernel when gridDim.z > 1.
 constexpr int SA_KN = 32;      // keys per tile
 constexpr int SA_PST = 33;     // row stride of the fp32 weight tiles (words)
-constexpr int SA_WST = 40;     // row stride of the bf16 mixed-weight / transposed-key tiles (elements)
+constexpr int SA_WST = 40;     // row stride of the bf16 mixed-weight tiles (elements)
 
 template <int NHW, int DS>
-__global__ void __launch_bounds__(256) sigattn_prefill_kernel(ktx_sigattn_config c, const float* __restrict__ q,
-                                                              const bf16_t* __restrict__ kcache, const float* __restrict__ kinv,
-                                                              const int32_t* __restrict__ q_indptr, const int32_t* __restrict__ pos0,
-                                                              const int32_t* __restrict__ page_indptr,
-                                                              const int32_t* __restrict__ page_indices, const float* __restrict__ pb,
-                                                              const float* __restrict__ talk, bf16_t* __restrict__ out) {
+__global__ void __launch_bounds__(256) sigattn_mfma_kernel(ktx_sigattn_config c, int T, const float* __restrict__ q,
+                                                           const bf16_t* __restrict__ kcache, const float* __restrict__ kinv,
+                                                           const int32_t* __restrict__ q_indptr, const int32_t* __restrict__ pos0,
+                                                           const int32_t* __restrict__ page_indptr,
+                                                           const int32_t* __restrict__ page_indices, const float* __restrict__ pb,
+                                                           const float* __restrict__ talk, float* __restrict__ partial,
+                                                           bf16_t* __restrict__ out) {
   extern __shared__ __attribute__((aligned(16))) unsigned char sa_lds[];
   constexpr int D = DS * 32;
   const int H = c.heads, G = c.kv_heads, rep = H / G, GD = G * D, HD = H * D;
   const int KST = GD + 8;
   bf16_t* ks = reinterpret_cast<bf16_t*>(sa_lds);                       // [32][KST]
-  bf16_t* vt = ks + SA_KN * KST;                                         // [GD][40]   transposed key tile
-  bf16_t* wm = vt + (size_t)GD * SA_WST;                                 // [H][16][40] mixed weights
+  bf16_t* wm = ks + SA_KN * KST;                                         // [H][16][40] mixed weights
   float* ps = reinterpret_cast<float*>(wm + (size_t)H * 16 * SA_WST);    // [H][16][33] weights
   float* kis = ps + (size_t)H * 16 * SA_PST;                             // [32][G]
   float* tks = kis + SA_KN * G;                                          // [H][H]
   const int b = blockIdx.y, tile = gridDim.x - 1 - blockIdx.x;            // long rows first
+  const int split = blockIdx.z, nsplit = gridDim.z;
   const int qb = q_indptr[b], qe = q_indptr[b + 1];
   const int row0 = qb + tile * 16;
   if (row0 >= qe) return;
@@ -538,17 +541,22 @@ __global__ void __launch_bounds__(256) sigattn_prefill_kernel(ktx_sigattn_config
   const int nrows = min(16, qe - row0);
   const int p0 = pos0[b] + tile * 16;                 // position of row 0 of the tile
   const int p_last = p0 + nrows - 1;
+  // this workgroup's key range, in whole tiles
+  const int ntiles = p_last / SA_KN + 1;
+  const int per = (ntiles + nsplit - 1) / nsplit;
+  const int jt0 = split * per, jt1 = min(ntiles, jt0 + per);
   const int32_t* pages = page_indices + page_indptr[b];
   for (int e = tid; e < H * H; e += 256) tks[e] = talk[e];
+  const int h0 = wave * NHW;
   // Q fragments (A operand: row = l16, k = ds*32 + lq*8 ..)
   sq_v8bf qf[NHW][DS];
 #pragma unroll
   for (int u = 0; u < NHW; u++) {
-    const int g = wave + 4 * u;
+    const int g = h0 + u;
 #pragma unroll
     for (int ds = 0; ds < DS; ds++) {
       uint4 pk = {0u, 0u, 0u, 0u};
-      if (g < H && l16 < nrows) {
+      if (g < H && l16 < nrows && jt0 < jt1) {
         const float* src = q + (size_t)(row0 + l16) * HD + g * D + ds * 32 + lq * 8;
         const float4 a = *reinterpret_cast<const float4*>(src), bq = *reinterpret_cast<const float4*>(src + 4);
         pk.x = ktx_pk_bf16(a.x, a.y); pk.y = ktx_pk_bf16(a.z, a.w); pk.z = ktx_pk_bf16(bq.x, bq.y); pk.w = ktx_pk_bf16(bq.z, bq.w);
@@ -564,50 +572,49 @@ __global__ void __launch_bounds__(256) sigattn_prefill_kernel(ktx_sigattn_config
   float slope[NHW], bias[NHW];
 #pragma unroll
   for (int u = 0; u < NHW; u++) {
-    const int g = wave + 4 * u;
+    const int g = h0 + u;
     slope[u] = (g < H && c.slope_span != 0.f) ? exp2f(-c.slope_span * (float)(g + 1) / (float)H) : 0.f;
     bias[u] = g < H ? pb[g] : 0.f;
   }
-  const int chunks = GD / 8;                           // 16-byte pieces of one key row
-  for (int j0 = 0; j0 <= p_last; j0 += SA_KN) {
+  // all heads of this wavefront on one key head?  (wave-uniform)
+  const bool shared_kv = (h0 / rep) == ((min(h0 + NHW, H) - 1) / rep);
+  const int sj = tid >> 3, sx = (tid & 7) * 8;        // staging: 8 threads per key row, 16-byte pieces 64 elements apart
+  for (int jt = jt0; jt < jt1; jt++) {
+    const int j0 = jt * SA_KN;
     __syncthreads();
-    for (int e = tid; e < SA_KN * chunks; e += 256) {
-      const int jj = e / chunks, x = (e - jj * chunks) * 8;
-      const int j = j0 + jj;
-      uint4 v = {0u, 0u, 0u, 0u};
-      if (j <= p_last) {
-        const size_t r = (size_t)pages[j / c.page_size] * c.page_size + (j % c.page_size);
-        v = *reinterpret_cast<const uint4*>(kcache + r * GD + x);
+    {
+      const int j = j0 + sj;
+      const bool ok = j <= p_last;
+      const size_t r = ok ? (size_t)pages[j / c.page_size] * c.page_size + (j % c.page_size) : 0;
+      const bf16_t* src = kcache + r * GD;
+      for (int x = sx; x < GD; x += 64) {
+        uint4 v = {0u, 0u, 0u, 0u};
+        if (ok) v = *reinterpret_cast<const uint4*>(src + x);
+        *reinterpret_cast<uint4*>(ks + sj * KST + x) = v;
       }
-      *reinterpret_cast<uint4*>(ks + jj * KST + x) = v;
-      const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        vt[(size_t)(x + 2 * i) * SA_WST + jj] = (bf16_t)(w4[i] & 0xffffu);
-        vt[(size_t)(x + 2 * i + 1) * SA_WST + jj] = (bf16_t)(w4[i] >> 16);
-      }
-    }
-    for (int e = tid; e < SA_KN * G; e += 256) {
-      const int jj = e / G, g = e - jj * G, j = j0 + jj;
-      float v = 0.f;
-      if (j <= p_last) v = kinv[((size_t)pages[j / c.page_size] * c.page_size + (j % c.page_size)) * G + g];
-      kis[e] = v;
+      if ((tid & 7) == 0)
+        for (int g = 0; g < G; g++) kis[sj * G + g] = ok ? kinv[r * G + g] : 0.f;
     }
     __syncthreads();
     // scores -> weights (fp32) of this wavefront's heads
 #pragma unroll
-    for (int u = 0; u < NHW; u++) {
-      const int g = wave + 4 * u;
-      if (g < H) {
-        const int kg = g / rep;
+    for (int nt = 0; nt < 2; nt++) {
+      sq_v8bf kf[DS];
+      int kg_have = -1;
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++) {
+      for (int u = 0; u < NHW; u++) {
+        const int g = h0 + u;
+        if (g < H) {
+          const int kg = g / rep;
+          if (kg != kg_have) {
+#pragma unroll
+            for (int ds = 0; ds < DS; ds++)
+              kf[ds] = *reinterpret_cast<const sq_v8bf*>(ks + (nt * 16 + l16) * KST + kg * D + ds * 32 + lq * 8);
+            kg_have = kg;
+          }
           v4f acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int ds = 0; ds < DS; ds++) {
-            const sq_v8bf kf = *reinterpret_cast<const sq_v8bf*>(ks + (nt * 16 + l16) * KST + kg * D + ds * 32 + lq * 8);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[u][ds], kf, acc, 0, 0, 0);
-          }
+          for (int ds = 0; ds < DS; ds++) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[u][ds], kf[ds], acc, 0, 0, 0);
           const int jj = nt * 16 + l16, j = j0 + jj;
           const float ki = kis[jj * G + kg];
 #pragma unroll
@@ -621,8 +628,8 @@ __global__ void __launch_bounds__(256) sigattn_prefill_kernel(ktx_sigattn_config
       }
     }
     __syncthreads();
-    // head mixing (fp32), then bf16 for the value product
-    {
+    // head mixing (fp32), then bf16 for the value product; rows of the tile that do not exist are skipped (decode steps have one)
+    if (lq * 4 < nrows) {
       float wacc[NHW][8];
 #pragma unroll
       for (int u = 0; u < NHW; u++)
@@ -636,7 +643,7 @@ __global__ void __launch_bounds__(256) sigattn_prefill_kernel(ktx_sigattn_config
           for (int r = 0; r < 4; r++) pv[nt * 4 + r] = ps[(g * 16 + lq * 4 + r) * SA_PST + nt * 16 + l16];
 #pragma unroll
         for (int u = 0; u < NHW; u++) {
-          const int h = wave + 4 * u;
+          const int h = h0 + u;
           const float tk = h < H ? tks[h * H + g] : 0.f;
 #pragma unroll
           for (int x = 0; x < 8; x++) wacc[u][x] = fmaf(tk, pv[x], wacc[u][x]);
@@ -644,7 +651,7 @@ __global__ void __launch_bounds__(256) sigattn_prefill_kernel(ktx_sigattn_config
       }
 #pragma unroll
       for (int u = 0; u < NHW; u++) {
-        const int h = wave + 4 * u;
+        const int h = h0 + u;
         if (h < H) {
 #pragma unroll
           for (int nt = 0; nt < 2; nt++)
@@ -652,18 +659,40 @@ __global__ void __launch_bounds__(256) sigattn_prefill_kernel(ktx_sigattn_config
             for (int r = 0; r < 4; r++) wm[(h * 16 + lq * 4 + r) * SA_WST + nt * 16 + l16] = to_bf16_rne(wacc[u][nt * 4 + r]);
         }
       }
+    } else {
+#pragma unroll
+      for (int u = 0; u < NHW; u++) {
+        const int h = h0 + u;
+        if (h < H) {
+#pragma unroll
+          for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) wm[(h * 16 + lq * 4 + r) * SA_WST + nt * 16 + l16] = 0;
+        }
+      }
     }
     __syncthreads();
-    // O_h += W_h V
+    // O_h += W_h V: B operand = V[k = key lq*8 .. +8][n = d]: eight 2-byte reads down a column of the key tile
 #pragma unroll
-    for (int u = 0; u < NHW; u++) {
-      const int h = wave + 4 * u;
-      if (h < H) {
-        const int kg = h / rep;
-        const sq_v8bf wf = *reinterpret_cast<const sq_v8bf*>(wm + (h * 16 + l16) * SA_WST + lq * 8);
+    for (int dn = 0; dn < DS * 2; dn++) {
+      sq_v8bf vf;
+      int kg_have = -1;
 #pragma unroll
-        for (int dn = 0; dn < DS * 2; dn++) {
-          const sq_v8bf vf = *reinterpret_cast<const sq_v8bf*>(vt + (size_t)(kg * D + dn * 16 + l16) * SA_WST + lq * 8);
+      for (int u = 0; u < NHW; u++) {
+        const int h = h0 + u;
+        if (h < H) {
+          const int kg = shared_kv ? h0 / rep : h / rep;
+          if (kg != kg_have) {
+            const bf16_t* col = ks + (size_t)(lq * 8) * KST + kg * D + dn * 16 + l16;
+            uint4 pk;
+            pk.x = (uint32_t)col[0] | ((uint32_t)col[KST] << 16);
+            pk.y = (uint32_t)col[2 * KST] | ((uint32_t)col[3 * KST] << 16);
+            pk.z = (uint32_t)col[4 * KST] | ((uint32_t)col[5 * KST] << 16);
+            pk.w = (uint32_t)col[6 * KST] | ((uint32_t)col[7 * KST] << 16);
+            vf = __builtin_bit_cast(sq_v8bf, pk);
+            kg_have = kg;
+          }
+          const sq_v8bf wf = *reinterpret_cast<const sq_v8bf*>(wm + (h * 16 + l16) * SA_WST + lq * 8);
           o[u][dn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, vf, o[u][dn], 0, 0, 0);
         }
       }
@@ -671,22 +700,26 @@ __global__ void __launch_bounds__(256) sigattn_prefill_kernel(ktx_sigattn_config
   }
 #pragma unroll
   for (int u = 0; u < NHW; u++) {
-    const int h = wave + 4 * u;
+    const int h = h0 + u;
     if (h < H) {
 #pragma unroll
       for (int dn = 0; dn < DS * 2; dn++)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           const int i = lq * 4 + r;
-          if (i < nrows) out[(size_t)(row0 + i) * HD + h * D + dn * 16 + l16] = to_bf16_rne(o[u][dn][r]);
+          if (i < nrows) {
+            const size_t e = (size_t)(row0 + i) * HD + h * D + dn * 16 + l16;
+            if (nsplit > 1) partial[(size_t)split * T * HD + e] = o[u][dn][r];
+            else out[e] = to_bf16_rne(o[u][dn][r]);
+          }
         }
     }
   }
 }
 
-size_t sigattn_prefill_lds(const ktx_sigattn_config& c) {
+size_t sigattn_mfma_lds(const ktx_sigattn_config& c) {
   const size_t GD = (size_t)c.kv_heads * c.dim, H = c.heads;
-  return SA_KN * (GD + 8) * 2 + GD * SA_WST * 2 + H * 16 * SA_WST * 2 + H * 16 * SA_PST * 4 + SA_KN * c.kv_heads * 4 + H * H * 4;
+  return SA_KN * (GD + 8) * 2 + H * 16 * SA_WST * 2 + H * 16 * SA_PST * 4 + SA_KN * c.kv_heads * 4 + H * H * 4;
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -916,27 +949,29 @@ int ktx_sigattn_forward(const ktx_sigattn_config* cfg, int T, const float* d_q, 
 
 int ktx_sigattn_prefill_eligible(const ktx_sigattn_config* c) {
   if (!c || sigattn_check(c, "ktx_sigattn_prefill_eligible")) return 0;
-  return c->cache_dtype == KTX_SEQ_BF16 && c->dim % 32 == 0 && c->dim <= 128 && c->heads <= 16 && sigattn_prefill_lds(*c) <= 150 * 1024;
+  return c->cache_dtype == KTX_SEQ_BF16 && c->dim % 32 == 0 && c->dim <= 128 && c->heads <= 16 && sigattn_mfma_lds(*c) <= 150 * 1024;
 }
 
-int ktx_sigattn_prefill(const ktx_sigattn_config* cfg, int B, int max_q_len, const float* d_q, const void* d_kcache,
+int ktx_sigattn_prefill(const ktx_sigattn_config* cfg, int B, int T, int max_q_len, const float* d_q, const void* d_kcache,
                         const float* d_kinv, const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_page_indptr,
-                        const int32_t* d_page_indices, const float* d_pb, const float* d_talk, void* d_out, ktx_stream_t stream) {
+                        const int32_t* d_page_indices, const float* d_pb, const float* d_talk, int nsplit, float* d_partial,
+                        void* d_out, ktx_stream_t stream) {
   KTX_REQUIRE(ktx_sigattn_prefill_eligible(cfg), "ktx_sigattn_prefill: needs a bf16 cache, dim % 32 == 0, dim <= 128, heads <= 16");
-  KTX_REQUIRE(B >= 0 && max_q_len >= 0 && d_q && d_kcache && d_kinv && d_q_indptr && d_pos0 && d_page_indptr && d_page_indices && d_pb &&
-                  d_talk && d_out, "ktx_sigattn_prefill: null pointer");
-  KTX_REQUIRE(B <= 65535, "ktx_sigattn_prefill: at most 65535 requests a call");
-  if (B == 0 || max_q_len == 0) return 0;
+  KTX_REQUIRE(B >= 0 && T >= 0 && max_q_len >= 0 && d_q && d_kcache && d_kinv && d_q_indptr && d_pos0 && d_page_indptr && d_page_indices &&
+                  d_pb && d_talk && d_out, "ktx_sigattn_prefill: null pointer");
+  KTX_REQUIRE(B <= 65535 && nsplit >= 1 && nsplit <= 65535 && (nsplit == 1 || d_partial),
+              "ktx_sigattn_prefill: at most 65535 requests and key ranges a call; scratch when nsplit > 1");
+  if (B == 0 || max_q_len == 0 || T == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
   const ktx_sigattn_config& c = *cfg;
-  const dim3 grid((max_q_len + 15) / 16, B);
-  const size_t lds = sigattn_prefill_lds(c);
+  const dim3 grid((max_q_len + 15) / 16, B, nsplit);
+  const size_t lds = sigattn_mfma_lds(c);
   const int nhw = (c.heads + 3) / 4, ds = c.dim / 32;
 #define KTX_SP_GO(NHW, DS)                                                                                                   \
   do {                                                                                                                       \
-    KTX_HIP(ktx_set_max_lds((const void*)sigattn_prefill_kernel<NHW, DS>, 160 * 1024));                                      \
-    sigattn_prefill_kernel<NHW, DS><<<grid, 256, lds, st>>>(c, d_q, (const bf16_t*)d_kcache, d_kinv, d_q_indptr, d_pos0,     \
-                                                            d_page_indptr, d_page_indices, d_pb, d_talk, (bf16_t*)d_out);    \
+    KTX_HIP(ktx_set_max_lds((const void*)sigattn_mfma_kernel<NHW, DS>, 160 * 1024));                                         \
+    sigattn_mfma_kernel<NHW, DS><<<grid, 256, lds, st>>>(c, T, d_q, (const bf16_t*)d_kcache, d_kinv, d_q_indptr, d_pos0,     \
+                                                         d_page_indptr, d_page_indices, d_pb, d_talk, d_partial, (bf16_t*)d_out); \
   } while (0)
 #define KTX_SP_DS(NHW)                                                          \
   do {                                                                          \
@@ -952,6 +987,11 @@ int ktx_sigattn_prefill(const ktx_sigattn_config* cfg, int B, int max_q_len, con
 #undef KTX_SP_DS
 #undef KTX_SP_GO
   KTX_HIP(hipGetLastError());
+  if (nsplit > 1) {
+    const size_t n = (size_t)T * c.heads * c.dim;
+    sigattn_reduce_kernel<bf16_t><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(nsplit, n, d_partial, (bf16_t*)d_out);
+    KTX_HIP(hipGetLastError());
+  }
   return 0;
 }
 

@@ -20,7 +20,7 @@ from ktransformers_amd.operators.base_operator import BaseInjectedModule
 
 
 class KSigmoidTalkAttention(BaseInjectedModule):
-    PREFILL_MIN_Q = 16      # steps whose longest request brings at least this many tokens take the matrix-core kernel
+    TARGET_WORKGROUPS = 1024
 
     def __init__(self, key: str, gguf_loader, config, orig_module: nn.Module, prefill_device: str = "cuda", generate_device: str = "cuda",
                  **kwargs):
@@ -66,9 +66,12 @@ class KSigmoidTalkAttention(BaseInjectedModule):
         cfg = self._config(cache)
         kc, kinv = cache.k_caches[self.layer_idx], cache.k_inv[self.layer_idx]
         q = sigattn_prep(cfg, proj, q_off, k_off, self.w["q_norm"], self.w["k_norm"], self.eps, batch.positions, batch.cache_loc, kc, kinv)
-        if batch.max_q_len >= self.PREFILL_MIN_Q and self.compute_dtype == torch.bfloat16 and sigattn_prefill_eligible(cfg):
+        if self.compute_dtype == torch.bfloat16 and sigattn_prefill_eligible(cfg):
+            # matrix-core kernel: tiles of 16 query rows x key ranges, enough workgroups to fill the chip
+            tiles = batch.B * ((batch.max_q_len + 15) // 16)
+            nsplit = max(1, min(self.TARGET_WORKGROUPS // max(tiles, 1), (batch.max_kv_len + 63) // 64))
             a = sigattn_prefill(cfg, q, kc, kinv, batch.q_indptr, batch.pos0, batch.page_indptr, batch.page_indices, self.w["pb"],
-                                self.w["talk"], batch.max_q_len)
+                                self.w["talk"], batch.max_q_len, nsplit=nsplit)
             return dense_gemm(a, self.w["o"])
         a = sigattn_forward(cfg, q, kc, kinv, batch.tok_req, batch.positions, batch.page_indptr, batch.page_indices, self.w["pb"],
                             self.w["talk"], nsplit=batch.nsplit, out_dtype=self.compute_dtype)

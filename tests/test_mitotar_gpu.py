@@ -171,12 +171,12 @@ def test_sigmoid_attention_matrix_core_kernel(H, G, D, T):
     w_in = torch.cat([P["a.q"], P["a.k"]]).to(BF16).to(DEV)
     f = lambda n: P[n].float().to(DEV).contiguous()
 
-    def run(cache, plan, hs):
+    def run(cache, plan, hs, nsplit=1):
         fb = cache.plan(plan)
         proj = dense_gemm(torch.cat(hs).float().to(DEV), w_in)
         q = sigattn_prep(cfg, proj, 0, H * D, f("a.q.norm"), f("a.k.norm"), 1e-5, fb.positions, fb.cache_loc, cache.k_caches[0], cache.k_inv[0])
         return sigattn_prefill(cfg, q, cache.k_caches[0], cache.k_inv[0], fb.q_indptr, fb.pos0, fb.page_indptr, fb.page_indices,
-                               f("a.pb"), f("a.talk"), fb.max_q_len)
+                               f("a.pb"), f("a.talk"), fb.max_q_len, nsplit=nsplit)
 
     cache = KHybridCache([{"attn": (G, D), "rec": None}], 4096, max_requests=4, page_size=8, dtype=BF16, device=DEV)
     cache.admit("r")
@@ -185,7 +185,9 @@ def test_sigmoid_attention_matrix_core_kernel(H, G, D, T):
     cut = T // 2 + 1
     a = run(cache, [("s", cut), ("t", 3)], [h[:cut], h[:3]])            # two requests, then the rest of one as a second portion
     assert rel(a[:cut], ref[:cut]) < TOL[BF16] and rel(a[cut:], ref[:3]) < TOL[BF16]
-    assert rel(run(cache, [("s", T - cut)], [h[cut:]]), ref[cut:]) < TOL[BF16]
+    assert rel(run(cache, [("s", T - cut - 2)], [h[cut:T - 2]], nsplit=3), ref[cut:T - 2]) < TOL[BF16]      # key ranges shared by workgroups
+    for t in (T - 2, T - 1):                                                                             # decode steps, more ranges than tiles
+        assert rel(run(cache, [("s", 1)], [h[t:t + 1]], nsplit=5), ref[t:t + 1]) < TOL[BF16]
 
 
 def test_prompt_sized_products_take_the_library_gemm():
