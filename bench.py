@@ -1607,7 +1607,7 @@ def run_mitotar(args, dev):
         with contextlib.redirect_stdout(io.StringIO()):
             model, config, entry = load_model(cfg, dtype=torch.bfloat16, device=str(dev), loader=SeqRandomLoader(cfg, dev))
         cache = entry.make_cache(config, 8 * (ctx + 64) + T, 16, torch.bfloat16, str(dev))
-        eng = BatchEngine(model, cache)
+        eng = BatchEngine(model, cache, use_graph=not args.no_graph)
         g = torch.Generator().manual_seed(5)
         prompt = torch.randint(0, 32000, (T,), generator=g).tolist()
         state = {"pairs": 0, "keys": 0}
@@ -1629,12 +1629,14 @@ def run_mitotar(args, dev):
                 state.update(pairs=B * cache.seq_len(ids[0]), keys=B * cache.seq_len(ids[0]))
                 eng.step([{"id": r, "tokens": [7], "want": [0]} for r in ids])
             ms = timed_ms(decode, 20)
+            eng.use_graph = False           # the per-kernel pass brackets eager launches
             with SeqKernelTimer(lambda: (state["pairs"], state["keys"])) as kt:
                 decode()
+            eng.use_graph = not args.no_graph
             kv_bytes = n_layers * B * ctx * sz["kv_heads"] * sz["dim"] * 2
             res[f"decode_bs{B}"] = {"tok_s": round(B / ms * 1e3, 1), "ms_per_step": round(ms, 3),
                                     "frac_of_hbm_peak": round((params * 2 + kv_bytes) / (ms * 1e-3) / (HBM_PEAK_GBS * 1e9), 4),
-                                    "per_kernel": kt.table(ms), "graph": False}
+                                    "per_kernel": kt.table(ms), "graph": eng.use_graph}
             for r in ids:
                 cache.release(r)
         res["weights_GB"] = round(params * 2 / 1e9, 3)

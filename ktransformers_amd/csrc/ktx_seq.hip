@@ -32,6 +32,10 @@ __device__ __forceinline__ float block_sum256(float v, float* red) {
 }
 
 __device__ __forceinline__ float sigmoid_f32(float z) { return 1.0f / (1.0f + expf(-z)); }
+// v_exp_f32 + v_rcp_f32 (about 1 ulp each): the matrix-core attention kernel, whose operands are bf16 anyway
+__device__ __forceinline__ float sigmoid_fast(float z) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z));
+}
 __device__ __forceinline__ float gelu_tanh_f32(float z) {
   return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
@@ -306,24 +310,93 @@ __global__ void __launch_bounds__(256) sigattn_reduce_kernel(int nsplit, size_t 
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
-// mLSTM recurrence: workgroup = (request, head, 64 value columns); wavefront w owns the rows d = w*DPG .. of the state slice,
-// lane = value column.  State slice, normaliser rows and the running maximum live in registers for the whole call.
+// mLSTM, part 1: the gates of a request's new tokens and the running maximum, off the sequential path.  Workgroup = (request, head).
+//   z_i, z_f -> log gates i_t, f_t (soft cap, logsigmoid);  m_t = max(f_t + m_(t-1), i_t) is a scan of maps m -> max(m + L, Z), which
+//   compose associatively ((L1, Z1) then (L2, Z2) = (L1 + L2, max(Z1 + L2, Z2))): 256 tokens per round, a wave scan on shuffles and
+//   the four wave totals through LDS.  Written per token: a_t = exp(f_t + m_(t-1) - m_t), b_t = exp(i_t - m_t), e_t = exp(-m_t).
+__global__ void __launch_bounds__(256) mlstm_gates_kernel(ktx_mlstm_config c, const int32_t* __restrict__ q_indptr,
+                                                          const int32_t* __restrict__ pos0, const int32_t* __restrict__ slot,
+                                                          const float* __restrict__ proj, int64_t ldp, int i_off, int f_off,
+                                                          const float* __restrict__ ib, const float* __restrict__ fb,
+                                                          float* __restrict__ mg, float* __restrict__ gates) {
+  __shared__ float wl[4], wz[4], mlast[256 + 1];
+  __shared__ float m_carry;
+  const int N = c.heads;
+  const int b = blockIdx.x, hd = blockIdx.y, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int t0 = q_indptr[b], t1 = q_indptr[b + 1];
+  if (t1 <= t0) return;
+  const int sl = slot[b];
+  if (tid == 0) m_carry = pos0[b] == 0 ? 0.f : mg[(size_t)sl * N + hd];
+  const float bi = ib[hd], bf = fb[hd], cap = c.gate_cap;
+  for (int base = t0; base < t1; base += 256) {
+    const int t = base + tid;
+    const bool ok = t < t1;
+    float L = 0.f, Z = -INFINITY, zi = 0.f;
+    if (ok) {
+      const float* row = proj + (size_t)t * ldp;
+      zi = row[i_off + hd] + bi;
+      float zf = row[f_off + hd] + bf;
+      if (cap != 0.f) {
+        zi = cap * tanhf(zi / cap);
+        zf = cap * tanhf(zf / cap);
+      }
+      L = log_sigmoid_f32(zf);
+      Z = zi;
+    }
+    const float lf = L;
+    // inclusive scan inside the wavefront
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const float pl = __shfl_up(L, d, 64), pz = __shfl_up(Z, d, 64);
+      if (lane >= d) {
+        Z = fmaxf(pz + L, Z);
+        L = pl + L;
+      }
+    }
+    __syncthreads();                        // (m_carry of the previous round has been read by everyone)
+    if (lane == 63) {
+      wl[wave] = L;
+      wz[wave] = Z;
+    }
+    __syncthreads();
+    float m_in = m_carry;
+    for (int w = 0; w < wave; w++) m_in = fmaxf(m_in + wl[w], wz[w]);
+    const float m = fmaxf(m_in + L, Z);
+    mlast[tid + 1] = m;
+    if (tid == 0) mlast[0] = m_carry;
+    __syncthreads();
+    if (ok) {
+      const float m_prev = mlast[tid];
+      float* g = gates + ((size_t)t * N + hd) * 3;
+      g[0] = expf(lf + m_prev - m);
+      g[1] = expf(zi - m);
+      g[2] = expf(-m);
+    }
+    const int last = min(256, t1 - base) - 1;
+    __syncthreads();
+    if (tid == last) m_carry = m;
+  }
+  __syncthreads();
+  if (tid == 0) mg[(size_t)sl * N + hd] = m_carry;
+}
+
+// mLSTM, part 2: the state recurrence.  Workgroup = (request, head, 64 value columns); wavefront w owns the rows d = w*DPG .. of the
+// state slice, lane = value column; state slice and normaliser rows live in registers for the whole call.  Per token: the decay /
+// input factors from part 1, k and q of the wavefront's rows (wave-uniform loads), S = a S + (b k) v, partial S^T q and n . q, ONE
+// barrier, and the first wavefront adds the four partials and divides.
 template <int DPG>
 __global__ void __launch_bounds__(256) mlstm_fwd_kernel(ktx_mlstm_config c, const int32_t* __restrict__ q_indptr,
                                                         const int32_t* __restrict__ pos0, const int32_t* __restrict__ slot,
                                                         const float* __restrict__ proj, int64_t ldp, int q_off, int k_off,
-                                                        int v_off, int i_off, int f_off, const float* __restrict__ ib,
-                                                        const float* __restrict__ fb, float* __restrict__ Sg,
-                                                        float* __restrict__ ng, float* __restrict__ mg,
-                                                        float* __restrict__ o_raw) {
-  extern __shared__ float lds[];
+                                                        int v_off, const float* __restrict__ gates, float* __restrict__ Sg,
+                                                        float* __restrict__ ng, float* __restrict__ o_raw) {
+  __shared__ float red[2][4][64];
+  __shared__ float redn[2][4];
+  __shared__ __attribute__((aligned(16))) float qk[2][2][4 * DPG];      // [half][q | k][rows, zero beyond dim]
   const int N = c.heads, D = c.dim, V = c.vdim;
-  float* qs = lds;              // [2][D]
-  float* kss = qs + 2 * D;      // [2][D]
-  float* red = kss + 2 * D;     // [4][64] partial outputs
-  float* redn = red + 256;      // [4]
   const int b = blockIdx.x, hd = blockIdx.y, vs = blockIdx.z;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int v = vs * 64 + lane;
   const bool vok = v < V;
   const int t0 = q_indptr[b], t1 = q_indptr[b + 1];
@@ -340,73 +413,66 @@ __global__ void __launch_bounds__(256) mlstm_fwd_kernel(ktx_mlstm_config c, cons
     S[i] = (!fresh && d < D && vok) ? Sp[(size_t)d * V + v] : 0.f;
     nn[i] = (!fresh && d < D) ? np_[d] : 0.f;
   }
-  float m = fresh ? 0.f : mg[(size_t)sl * N + hd];
+  for (int e = tid; e < 2 * 2 * 4 * DPG; e += 256) (&qk[0][0][0])[e] = 0.f;
+  __syncthreads();
   const float qscale = 1.0f / sqrtf((float)D);
-  const float bi = ib[hd], bf = fb[hd], cap = c.gate_cap;
-  // the next token's inputs are requested a step ahead: their latency hides behind this token's update and barriers
-  float nq = 0.f, nk = 0.f, nv = 0.f, nzi = 0.f, nzf = 0.f;
+  // q and k of a token reach the wavefronts through LDS (one element per thread, broadcast reads); everything a token brings is
+  // requested a step ahead: while token t is computed, token t+1's q / k go into the other LDS half and token t+2's are in flight
+  float rq = 0.f, rk = 0.f, nv, na, nb, ne;
   {
     const float* row = proj + (size_t)t0 * ldp;
+    const float* g = gates + ((size_t)t0 * N + hd) * 3;
     if (tid < D) {
-      nq = row[q_off + hd * D + tid];
-      nk = row[k_off + hd * D + tid];
+      qk[0][0][tid] = row[q_off + hd * D + tid] * qscale;
+      qk[0][1][tid] = row[k_off + hd * D + tid];
     }
-    if (vok) nv = row[v_off + hd * V + v];
-    nzi = row[i_off + hd];
-    nzf = row[f_off + hd];
+    nv = vok ? row[v_off + hd * V + v] : 0.f;
+    na = g[0], nb = g[1], ne = g[2];
+    if (t0 + 1 < t1 && tid < D) {
+      const float* r1 = proj + (size_t)(t0 + 1) * ldp;
+      rq = r1[q_off + hd * D + tid];
+      rk = r1[k_off + hd * D + tid];
+    }
   }
+  __syncthreads();
   for (int t = t0; t < t1; t++) {
     const int buf = (t - t0) & 1;
-    float* qb = qs + buf * D;
-    float* kb = kss + buf * D;
-    const float cq = nq, ck = nk, vv = nv;
-    float zi = nzi + bi, zf = nzf + bf;
+    const float vv = nv, a = na, bb = nb, e = ne;
+    if (tid < D) {
+      qk[buf ^ 1][0][tid] = rq * qscale;
+      qk[buf ^ 1][1][tid] = rk;
+    }
     if (t + 1 < t1) {
       const float* row = proj + (size_t)(t + 1) * ldp;
-      if (tid < D) {
-        nq = row[q_off + hd * D + tid];
-        nk = row[k_off + hd * D + tid];
+      const float* g = gates + ((size_t)(t + 1) * N + hd) * 3;
+      nv = vok ? row[v_off + hd * V + v] : 0.f;
+      na = g[0], nb = g[1], ne = g[2];
+      if (t + 2 < t1 && tid < D) {
+        const float* r2 = proj + (size_t)(t + 2) * ldp;
+        rq = r2[q_off + hd * D + tid];
+        rk = r2[k_off + hd * D + tid];
       }
-      if (vok) nv = row[v_off + hd * V + v];
-      nzi = row[i_off + hd];
-      nzf = row[f_off + hd];
     }
-    if (tid < D) {
-      qb[tid] = cq * qscale;
-      kb[tid] = ck;
-    }
-    if (cap != 0.f) {
-      zi = cap * tanhf(zi / cap);
-      zf = cap * tanhf(zf / cap);
-    }
-    const float lf = log_sigmoid_f32(zf);
-    const float m_new = fmaxf(lf + m, zi);
-    const float a = expf(lf + m - m_new), bb = expf(zi - m_new);
-    m = m_new;
-    __syncthreads();
     float po = 0.f, pn = 0.f;
+    const float* qb = &qk[buf][0][d0];
+    const float* kb = &qk[buf][1][d0];
 #pragma unroll
     for (int i = 0; i < DPG; i++) {
-      const int d = d0 + i;
-      if (d < D) {
-        const float kd = kb[d], qd = qb[d];
-        const float bk = bb * kd;
-        S[i] = a * S[i] + bk * vv;
-        nn[i] = a * nn[i] + bk;
-        po += S[i] * qd;
-        pn += nn[i] * qd;
-      }
+      const float bk = bb * kb[i], qd = qb[i];
+      S[i] = a * S[i] + bk * vv;
+      nn[i] = a * nn[i] + bk;
+      po += S[i] * qd;
+      pn += nn[i] * qd;
     }
-    red[wave * 64 + lane] = po;
-    if (lane == 0) redn[wave] = pn;
+    red[buf][wave][lane] = po;
+    if (lane == 0) redn[buf][wave] = pn;
     __syncthreads();
     if (wave == 0 && vok) {
-      const float num = ((red[lane] + red[64 + lane]) + red[128 + lane]) + red[192 + lane];
-      const float nq = ((redn[0] + redn[1]) + redn[2]) + redn[3];
-      const float den = fmaxf(fabsf(nq), expf(-m)) + c.denom_eps;
-      o_raw[(size_t)t * N * V + hd * V + v] = num / den;
+      const float num = ((red[buf][0][lane] + red[buf][1][lane]) + red[buf][2][lane]) + red[buf][3][lane];
+      const float nqd = ((redn[buf][0] + redn[buf][1]) + redn[buf][2]) + redn[buf][3];
+      o_raw[(size_t)t * N * V + hd * V + v] = num / (fmaxf(fabsf(nqd), e) + c.denom_eps);
     }
-    // (the next token stages into the other q / k buffer; `red` is rewritten only behind the next token's first barrier)
+    // (the next token writes the other halves of `red` and `qk`; these halves are rewritten only behind the next barrier)
   }
 #pragma unroll
   for (int i = 0; i < DPG; i++) {
@@ -416,7 +482,6 @@ __global__ void __launch_bounds__(256) mlstm_fwd_kernel(ktx_mlstm_config c, cons
       if (vs == 0 && lane == 0) np_[d] = nn[i];
     }
   }
-  if (vs == 0 && tid == 0) mg[(size_t)sl * N + hd] = m;
 }
 
 template <typename OT>
@@ -621,7 +686,7 @@ __global__ void __launch_bounds__(256) sigattn_mfma_kernel(ktx_sigattn_config c,
           for (int r = 0; r < 4; r++) {
             const int i = lq * 4 + r, pi = p0 + i;
             float w = 0.f;
-            if (i < nrows && j <= pi) w = sigmoid_f32(acc[r] * ki - slope[u] * (float)(pi - j) + bias[u]);
+            if (i < nrows && j <= pi) w = sigmoid_fast(acc[r] * ki - slope[u] * (float)(pi - j) + bias[u]);
             ps[(g * 16 + i) * SA_PST + jj] = w;
           }
         }
@@ -1009,10 +1074,10 @@ int ktx_gelu_tanh(size_t n, void* d_y, int dtype, ktx_stream_t stream) {
 
 int ktx_mlstm_forward(const ktx_mlstm_config* cfg, int B, const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_slot,
                       const float* d_proj, int64_t ldp, int q_off, int k_off, int v_off, int i_off, int f_off, const float* d_ib,
-                      const float* d_fb, float* d_S, float* d_n, float* d_m, float* d_o_raw, ktx_stream_t stream) {
+                      const float* d_fb, float* d_S, float* d_n, float* d_m, float* d_gates, float* d_o_raw, ktx_stream_t stream) {
   KTX_REQUIRE(cfg && cfg->heads > 0 && cfg->dim > 0 && cfg->vdim > 0, "ktx_mlstm_forward: heads, dim, vdim must be positive");
   KTX_REQUIRE(cfg->dim <= 256, "ktx_mlstm_forward: dim must be <= 256 (a wavefront keeps dim / 4 state rows in registers)");
-  KTX_REQUIRE(B >= 0 && d_q_indptr && d_pos0 && d_slot && d_proj && d_ib && d_fb && d_S && d_n && d_m && d_o_raw,
+  KTX_REQUIRE(B >= 0 && d_q_indptr && d_pos0 && d_slot && d_proj && d_ib && d_fb && d_S && d_n && d_m && d_gates && d_o_raw,
               "ktx_mlstm_forward: null pointer");
   const int64_t need = std::max(std::max((int64_t)q_off + cfg->heads * cfg->dim, (int64_t)k_off + cfg->heads * cfg->dim),
                                 std::max((int64_t)v_off + cfg->heads * cfg->vdim, (int64_t)std::max(i_off, f_off) + cfg->heads));
@@ -1022,11 +1087,12 @@ int ktx_mlstm_forward(const ktx_mlstm_config* cfg, int B, const int32_t* d_q_ind
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid(B, cfg->heads, (cfg->vdim + 63) / 64);
   KTX_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "ktx_mlstm_forward: too many heads / value columns");
-  const size_t lds = (4 * (size_t)cfg->dim + 256 + 4) * sizeof(float);
+  mlstm_gates_kernel<<<dim3(B, cfg->heads), 256, 0, st>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_proj, ldp, i_off, f_off, d_ib, d_fb, d_m,
+                                                          d_gates);
   const int dpg = (cfg->dim + 3) / 4;
-#define KTX_ML_GO(DPG)                                                                                                          \
-  mlstm_fwd_kernel<DPG><<<grid, 256, lds, st>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_proj, ldp, q_off, k_off, v_off, i_off, f_off, \
-                                                d_ib, d_fb, d_S, d_n, d_m, d_o_raw)
+#define KTX_ML_GO(DPG)                                                                                                       \
+  mlstm_fwd_kernel<DPG><<<grid, 256, 0, st>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_proj, ldp, q_off, k_off, v_off, d_gates, d_S, \
+                                              d_n, d_o_raw)
   if (dpg <= 4) KTX_ML_GO(4);
   else if (dpg <= 8) KTX_ML_GO(8);
   else if (dpg <= 16) KTX_ML_GO(16);

@@ -200,6 +200,7 @@ class KHybridCache:
         self.free_pages = list(range(self.num_pages - 1, -1, -1))
         self.free_slots = list(range(self.max_requests - 1, -1, -1))
         self.requests: Dict[Any, dict] = {}
+        self.generation = 0          # bumped whenever the tensors are re-allocated (captured graphs hold their addresses)
 
     # ---- allocation ------------------------------------------------------------------------------------------------
     def admit(self, rid) -> None:
@@ -235,6 +236,7 @@ class KHybridCache:
         self.S, self.n, self.m = [grow(t) for t in self.S], [grow(t) for t in self.n], [grow(t) for t in self.m]
         self.free_slots.extend(range(self.max_requests + extra - 1, self.max_requests - 1, -1))
         self.max_requests += extra
+        self.generation += 1
 
     def _add_pages(self, extra: int) -> None:
         rows = extra * self.page_size
@@ -243,36 +245,41 @@ class KHybridCache:
         self.free_pages.extend(range(self.num_pages + extra - 1, self.num_pages - 1, -1))
         self.num_pages += extra
         self.max_cache_len = self.num_pages * self.page_size
+        self.generation += 1
 
-    def plan(self, entries, target_workgroups: int = 1024, keys_per_split: int = 128) -> ForwardBatch:
-        """entries: [(request id, number of new tokens)], in batch order.  Grows each request's page list, advances its length and
-        returns the step's ForwardBatch (host lists -> device tensors, one copy each)."""
+    def plan_lists(self, entries) -> dict:
+        """The host half of plan(): grows each request's page list, advances its length and returns the step's metadata as python
+        lists (same field names as ForwardBatch) — what a captured decode graph copies into its static buffers."""
         ps = self.page_size
-        positions, tok_req, cache_loc, q_indptr, pos0, slot, page_indptr, page_indices = [], [], [], [0], [], [], [0], []
+        d = {k: [] for k in ("positions", "tok_req", "cache_loc", "pos0", "slot", "page_indices")}
+        d["q_indptr"], d["page_indptr"] = [0], [0]
         max_q = max_kv = 0
         for b, (rid, n_new) in enumerate(entries):
             r = self.requests[rid]
             self._grow(r, n_new)
-            start = r["len"]
-            pages = r["pages"]
+            start, pages = r["len"], r["pages"]
             for p in range(start, start + n_new):
-                positions.append(p)
-                tok_req.append(b)
-                cache_loc.append(pages[p // ps] * ps + p % ps)
+                d["positions"].append(p)
+                d["tok_req"].append(b)
+                d["cache_loc"].append(pages[p // ps] * ps + p % ps)
             r["len"] = start + n_new
-            q_indptr.append(q_indptr[-1] + n_new)
-            pos0.append(start)
-            slot.append(r["slot"])
-            page_indices.extend(pages)
-            page_indptr.append(len(page_indices))
+            d["q_indptr"].append(d["q_indptr"][-1] + n_new)
+            d["pos0"].append(start)
+            d["slot"].append(r["slot"])
+            d["page_indices"].extend(pages)
+            d["page_indptr"].append(len(d["page_indices"]))
             max_q, max_kv = max(max_q, n_new), max(max_kv, r["len"])
-        T = len(positions)
-        dev = self.device
-        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
-        nsplit = max(1, min(target_workgroups // max(T, 1), (max_kv + keys_per_split - 1) // keys_per_split))
-        return ForwardBatch(T=T, B=len(entries), positions=i32(positions), tok_req=i32(tok_req), cache_loc=i32(cache_loc),
-                            q_indptr=i32(q_indptr), pos0=i32(pos0), slot=i32(slot), page_indptr=i32(page_indptr),
-                            page_indices=i32(page_indices), max_q_len=max_q, max_kv_len=max_kv, nsplit=nsplit)
+        d.update(T=len(d["positions"]), B=len(entries), max_q_len=max_q, max_kv_len=max_kv)
+        return d
+
+    def plan(self, entries, target_workgroups: int = 1024, keys_per_split: int = 128) -> ForwardBatch:
+        """entries: [(request id, number of new tokens)], in batch order -> the step's ForwardBatch (plan_lists on the device)."""
+        d = self.plan_lists(entries)
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=self.device)
+        nsplit = max(1, min(target_workgroups // max(d["T"], 1), (d["max_kv_len"] + keys_per_split - 1) // keys_per_split))
+        return ForwardBatch(T=d["T"], B=d["B"], max_q_len=d["max_q_len"], max_kv_len=d["max_kv_len"], nsplit=nsplit,
+                            **{k: i32(d[k]) for k in ("positions", "tok_req", "cache_loc", "q_indptr", "pos0", "slot", "page_indptr",
+                                                      "page_indices")})
 
     # ---- the single-request view util.generate.prefill_and_generate drives (one sequence, positions given by the caller) --------
     SINGLE = "__single__"

@@ -13,10 +13,85 @@ import torch
 from ktransformers_amd.util.generate import sample_next_token
 
 
+class _DecodeGraph:
+    """One captured decode step (one token per request) for a batch of B requests: the step's metadata lives in ONE static int32
+    device buffer whose slices are the ForwardBatch's tensors; a step fills a pinned host copy, sends it with one transfer and
+    replays.  Valid while B, the page-list capacity, the key-range split and the cache's tensors stay what they were."""
+    FIELDS = ("tokens", "positions", "tok_req", "cache_loc", "pos0", "slot", "q_indptr", "page_indptr", "page_indices")
+
+    def __init__(self, engine, B: int, page_cap: int, nsplit: int, max_kv_len: int):
+        from ktransformers_amd.models.custom_cache import ForwardBatch
+        self.B, self.page_cap, self.nsplit = B, page_cap, nsplit
+        sizes = dict(tokens=B, positions=B, tok_req=B, cache_loc=B, pos0=B, slot=B, q_indptr=B + 1, page_indptr=B + 1, page_indices=page_cap)
+        self.offsets, at = {}, 0
+        for k in self.FIELDS:
+            self.offsets[k] = (at, sizes[k])
+            at += (sizes[k] + 3) // 4 * 4                 # 16-byte aligned slices
+        dev = engine.device
+        self.host = torch.zeros(at, dtype=torch.int32, pin_memory=True)
+        self.meta = torch.zeros(at, dtype=torch.int32, device=dev)
+        v = {k: self.meta[o:o + n] for k, (o, n) in self.offsets.items()}
+        self.tokens = v["tokens"]
+        self.batch = ForwardBatch(T=B, B=B, max_q_len=1, max_kv_len=max_kv_len, nsplit=nsplit,
+                                  **{k: v[k] for k in self.FIELDS if k != "tokens"})
+        self.graph, self.logits = None, None
+
+    def fill(self, d: dict, tokens) -> None:
+        h = self.host
+        for k in self.FIELDS:
+            o, n = self.offsets[k]
+            vals = tokens if k == "tokens" else d[k]
+            h[o:o + len(vals)] = torch.tensor(vals, dtype=torch.int32)
+        self.meta.copy_(h, non_blocking=True)
+
+    def capture(self, engine) -> None:
+        cache, model, dev = engine.cache, engine.model, engine.device
+        # the warm-up runs advance the recurrent state of the batch's slots: put it back afterwards (appending the same key rows
+        # again changes nothing)
+        keep = [(t, t.clone()) for group in (cache.S, cache.n, cache.m) for t in group if t is not None]
+        stream = torch.cuda.Stream(device=dev)
+        stream.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(stream):
+            for _ in range(2):
+                model(self.tokens, None, cache, batch=self.batch)
+        torch.cuda.current_stream(dev).wait_stream(stream)
+        torch.cuda.synchronize(dev)
+        for t, saved in keep:
+            t.copy_(saved)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, stream=stream):
+            self.logits = model(self.tokens, None, cache, batch=self.batch)
+        torch.cuda.synchronize(dev)
+
+
 class BatchEngine:
-    def __init__(self, model, cache):
+    def __init__(self, model, cache, use_graph: bool = False):
+        """use_graph: steps that bring exactly one token for every request (decode steps) replay a captured HIP graph."""
         self.model, self.cache = model, cache
         self.device = cache.device
+        self.use_graph = use_graph
+        self._graphs: dict = {}
+        self._graph_generation = cache.generation
+
+    def _decode_graph_step(self, plan, tokens, rows):
+        d = self.cache.plan_lists(plan)
+        if self._graph_generation != self.cache.generation:          # the cache re-allocated its tensors
+            self._graphs.clear()
+            self._graph_generation = self.cache.generation
+        B = d["B"]
+        page_cap = (len(d["page_indices"]) + 63) // 64 * 64
+        kv_bucket = (d["max_kv_len"] + 1023) // 1024 * 1024
+        nsplit = max(1, min(1024 // B, kv_bucket // 128))
+        key = (B, page_cap, nsplit)
+        g = self._graphs.get(key)
+        fresh = g is None
+        if fresh:
+            g = self._graphs[key] = _DecodeGraph(self, B, page_cap, nsplit, kv_bucket)
+        g.fill(d, tokens)
+        if fresh:
+            g.capture(self)
+        g.graph.replay()
+        return g.logits[torch.tensor(rows, dtype=torch.long, device=self.device)] if rows else None
 
     @torch.no_grad()
     def step(self, entries, end=()):
@@ -37,7 +112,9 @@ class BatchEngine:
                 rows.append(base + w)
             base += n
         logits = None
-        if plan:
+        if plan and self.use_graph and all(n == 1 for _, n in plan) and all(self.cache.seq_len(r) > 0 for r, _ in plan):
+            logits = self._decode_graph_step(plan, tokens, rows)
+        elif plan:
             batch = self.cache.plan(plan)
             ids = torch.tensor(tokens, dtype=torch.int32, device=self.device)
             if rows:

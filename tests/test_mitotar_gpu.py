@@ -419,3 +419,33 @@ def test_greedy_generation_through_both_loops(dtype):
         ids = torch.tensor([prompts["p"]], dtype=torch.int64, device=DEV)
         toks = prefill_and_generate(model, ids, c1, max_new_tokens=n_new, use_cuda_graph=use_graph, chunk_size=8).tolist()
         assert toks == out["p"], (use_graph, toks, out["p"])
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_captured_decode_steps_equal_eager_ones(dtype):
+    """Decode steps of a batch replayed from a captured HIP graph, with eager work (another request's prompt) and a change of the
+    batch between replays: every replay against the eager engine's logits and against the plain statement."""
+    from ktransformers_amd.util.batch_engine import BatchEngine
+    cfg = R.make_config(**CONFIGS["mfma"])
+    model, cache, P = build(cfg, 21, dtype, page_size=16)
+    _, cache2, _ = build(cfg, 21, dtype, page_size=16)
+    eager, graphed = BatchEngine(model, cache2), BatchEngine(model, cache, use_graph=True)
+    reqs = {"a": tokens_of(cfg, 30, 1), "b": tokens_of(cfg, 9, 2)}
+    cont = {r: tokens_of(cfg, 12, 30 + i) for i, r in enumerate(reqs)}
+    ref = {r: R.forward(P, cfg, reqs[r] + cont[r]) for r in reqs}
+    for eng in (eager, graphed):
+        eng.step([{"id": r, "tokens": t, "want": []} for r, t in reqs.items()])
+    live = list(reqs)
+    for k in range(12):
+        entries = [{"id": r, "tokens": [cont[r][k]], "want": [0]} for r in live]
+        end = ["b"] if k == 6 else []
+        le, lg = eager.step(entries, end), graphed.step(entries, end)
+        assert rows_rel(lg, le) < (1e-5 if dtype == F32 else 2e-2), k
+        for i, r in enumerate(live):
+            p = len(reqs[r]) + k
+            assert rows_rel(lg[i:i + 1], ref[r][p:p + 1]) < (TOL[dtype] if dtype == F32 else 0.12), (k, r)
+        live = [r for r in live if r not in end]
+        if k == 3:      # eager work between two replays
+            for eng in (eager, graphed):
+                eng.step([{"id": "c", "tokens": tokens_of(cfg, 20, 9), "want": [19]}], ["c"])
+    assert len(graphed._graphs) >= 2
