@@ -562,6 +562,52 @@ __global__ void __launch_bounds__(256) dense_gemv_kernel(int M, int N, int K, co
   }
 }
 
+// decode-sized GEMM on the matrix cores (M <= 16, bf16 weights, K % 32 == 0): workgroup = 16 weight rows, its four wavefronts take a
+// quarter of K each; a lane streams ITS weight row's 16-byte pieces straight from memory into the B operand (no LDS on the weight
+// path), the activation rows (few, L2-resident) fill the A operand; partial tiles meet in LDS.
+template <typename AT, typename YT>
+__global__ void __launch_bounds__(256) dense_gemv_mfma_kernel(int M, int N, int K, const AT* __restrict__ A, int64_t lda,
+                                                              const bf16_t* __restrict__ W, YT* __restrict__ Y, int64_t ldy, int act) {
+  __shared__ float red[4][64][4];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
+  const int n = blockIdx.x * 16 + l16;
+  const int steps = K / 32, per = (steps + 3) / 4;
+  const int s0 = wave * per, s1 = min(steps, s0 + per);
+  const bf16_t* wrow = W + (size_t)min(n, N - 1) * K + lq * 8;
+  const AT* arow = A + (size_t)min(l16, M - 1) * lda + lq * 8;
+  const bool aok = l16 < M, wok = n < N;
+  v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int st = s0; st < s1; st++) {
+    const int k = st * 32;
+    uint4 wv = *reinterpret_cast<const uint4*>(wrow + k);
+    uint4 av;
+    if constexpr (sizeof(AT) == 4) {
+      const float4 a0 = *reinterpret_cast<const float4*>(arow + k), a1 = *reinterpret_cast<const float4*>(arow + k + 4);
+      av.x = ktx_pk_bf16(a0.x, a0.y); av.y = ktx_pk_bf16(a0.z, a0.w); av.z = ktx_pk_bf16(a1.x, a1.y); av.w = ktx_pk_bf16(a1.z, a1.w);
+    } else {
+      av = *reinterpret_cast<const uint4*>(arow + k);
+    }
+    if (!aok) av = uint4{0u, 0u, 0u, 0u};
+    if (!wok) wv = uint4{0u, 0u, 0u, 0u};
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sq_v8bf, av), __builtin_bit_cast(sq_v8bf, wv), acc, 0, 0, 0);
+  }
+#pragma unroll
+  for (int r = 0; r < 4; r++) red[wave][lane][r] = acc[r];
+  __syncthreads();
+  if (wave == 0 && wok) {
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int m = lq * 4 + r;
+      if (m < M) {
+        float v = ((red[0][lane][r] + red[1][lane][r]) + red[2][lane][r]) + red[3][lane][r];
+        if (act == KTX_ACT_GELU_TANH) v = gelu_tanh_f32(v);
+        st_elem(Y, (size_t)m * ldy + n, v);
+      }
+    }
+  }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256) gelu_tanh_kernel(size_t n, T* __restrict__ y) {
   const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -796,30 +842,73 @@ __global__ void __launch_bounds__(256) rms_combine_kernel(int W, const float* __
                                                           float* __restrict__ xres, const int32_t* __restrict__ rows,
                                                           OT* __restrict__ out) {
   __shared__ float red[4];
+  constexpr int RMAX = 16;                  // rows up to 256 * 16 elements stay in registers; longer ones are re-read
   const int t = blockIdx.x, tid = threadIdx.x;
   const float* a = y1 + (size_t)(rows ? rows[t] : t) * W;
   const float* b = y2 ? y2 + (size_t)t * W : nullptr;
+  const bool in_regs = W <= 256 * RMAX;
+  float za[RMAX], zb[RMAX];
   float r1 = 1.f, r2 = 1.f;
+  if (in_regs) {
+#pragma unroll
+    for (int i = 0; i < RMAX; i++) {
+      const int e = tid + i * 256;
+      za[i] = e < W ? a[e] : 0.f;
+      zb[i] = (b && e < W) ? b[e] : 0.f;
+    }
+  }
   if (b) {
     float s1 = 0.f, s2 = 0.f;
-    for (int e = tid; e < W; e += 256) {
-      s1 += a[e] * a[e];
-      s2 += b[e] * b[e];
+    if (in_regs) {
+#pragma unroll
+      for (int i = 0; i < RMAX; i++) {
+        s1 += za[i] * za[i];
+        s2 += zb[i] * zb[i];
+      }
+    } else {
+      for (int e = tid; e < W; e += 256) {
+        s1 += a[e] * a[e];
+        s2 += b[e] * b[e];
+      }
     }
     s1 = block_sum256(s1, red);
     s2 = block_sum256(s2, red);
     r1 = 1.0f / sqrtf(s1 / (float)W + eps);
     r2 = 1.0f / sqrtf(s2 / (float)W + eps);
+    if (in_regs) {
+#pragma unroll
+      for (int i = 0; i < RMAX; i++) {
+        const int e = tid + i * 256;
+        if (e < W) za[i] = 0.5f * (za[i] * r1 * w1[e] + zb[i] * r2 * w2[e]);
+      }
+    }
   }
   float rz = 1.f;
   if (wn) {
     float sz = 0.f;
-    for (int e = tid; e < W; e += 256) {
-      const float z = b ? 0.5f * (a[e] * r1 * w1[e] + b[e] * r2 * w2[e]) : a[e];
-      sz += z * z;
+    if (in_regs) {
+#pragma unroll
+      for (int i = 0; i < RMAX; i++) sz += za[i] * za[i];
+    } else {
+      for (int e = tid; e < W; e += 256) {
+        const float z = b ? 0.5f * (a[e] * r1 * w1[e] + b[e] * r2 * w2[e]) : a[e];
+        sz += z * z;
+      }
     }
     sz = block_sum256(sz, red);
     rz = 1.0f / sqrtf(sz / (float)W + eps);
+  }
+  if (in_regs) {
+#pragma unroll
+    for (int i = 0; i < RMAX; i++) {
+      const int e = tid + i * 256;
+      if (e < W) {
+        const float r = wn ? za[i] * rz * (one_plus ? 1.0f + wn[e] : wn[e]) : za[i];
+        if (xres) xres[(size_t)t * W + e] += r;
+        else st_elem(out, (size_t)t * W + e, r);
+      }
+    }
+    return;
   }
   for (int e = tid; e < W; e += 256) {
     const float z = b ? 0.5f * (a[e] * r1 * w1[e] + b[e] * r2 * w2[e]) : a[e];
@@ -889,8 +978,22 @@ int ktx_dense_gemm(int M, int N, int K, const void* d_A, int a_dtype, int64_t ld
   KTX_REQUIRE(!(w_dtype == KTX_SEQ_F32 && a_dtype != KTX_SEQ_F32), "ktx_dense_gemm: an fp32 product needs fp32 activations");
   if (M == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
+  if (M <= 16 && ksplit == 1 && w_dtype == KTX_SEQ_BF16 && K % 32 == 0 && aligned16(d_W) && aligned16(d_A) &&
+      (lda * (a_dtype == KTX_SEQ_F32 ? 4 : 2)) % 16 == 0) {
+    const unsigned blocks = (unsigned)((N + 15) / 16);
+    if (a_dtype == KTX_SEQ_F32 && y_dtype == KTX_SEQ_F32)
+      dense_gemv_mfma_kernel<float, float><<<blocks, 256, 0, st>>>(M, N, K, (const float*)d_A, lda, (const bf16_t*)d_W, (float*)d_Y, ldy, act);
+    else if (a_dtype == KTX_SEQ_F32)
+      dense_gemv_mfma_kernel<float, bf16_t><<<blocks, 256, 0, st>>>(M, N, K, (const float*)d_A, lda, (const bf16_t*)d_W, (bf16_t*)d_Y, ldy, act);
+    else if (y_dtype == KTX_SEQ_F32)
+      dense_gemv_mfma_kernel<bf16_t, float><<<blocks, 256, 0, st>>>(M, N, K, (const bf16_t*)d_A, lda, (const bf16_t*)d_W, (float*)d_Y, ldy, act);
+    else
+      dense_gemv_mfma_kernel<bf16_t, bf16_t><<<blocks, 256, 0, st>>>(M, N, K, (const bf16_t*)d_A, lda, (const bf16_t*)d_W, (bf16_t*)d_Y, ldy, act);
+    KTX_HIP(hipGetLastError());
+    return 0;
+  }
   {
-    // decode-sized calls: the streaming kernel, when the activation rows fit the LDS
+    // decode-sized calls of any other shape or type: the streaming kernel, when the activation rows fit the LDS
     const size_t wsz0 = w_dtype == KTX_SEQ_F32 ? 4 : 2;
     const int mm = M <= 2 ? 2 : 8;
     const size_t lds = (size_t)mm * ((K + 7) & ~7) * wsz0;

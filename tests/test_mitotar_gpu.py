@@ -71,7 +71,7 @@ def test_embedding_with_sinusoid_positions(dtype, width, vocab):
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
-@pytest.mark.parametrize("M,N,K", [(1, 5, 7), (3, 64, 32), (70, 130, 100), (65, 17, 264), (128, 192, 64)])
+@pytest.mark.parametrize("M,N,K", [(1, 5, 7), (3, 64, 32), (70, 130, 100), (65, 17, 264), (128, 192, 64), (1, 200, 96), (8, 37, 256), (16, 64, 2048), (9, 5000, 320)])
 def test_dense_gemm_any_shape(dtype, M, N, K):
     from ktransformers_amd._native_seq import dense_gemm
     g = torch.Generator().manual_seed(M * 1000 + N)
@@ -89,7 +89,7 @@ def test_dense_gemm_any_shape(dtype, M, N, K):
 def test_norm_glue_forms():
     from ktransformers_amd._native_seq import rms_combine
     g = torch.Generator().manual_seed(3)
-    for W in (48, 37, 300):
+    for W in (48, 37, 300, 5000):
         y1, y2, x = (torch.randn(5, W, generator=g) for _ in range(3))
         w1, w2, wn = (torch.randn(W, generator=g) for _ in range(3))
         eps = 1e-3
