@@ -639,8 +639,8 @@ __global__ void __launch_bounds__(256) sigattn_mfma_kernel(ktx_sigattn_config c,
   const int H = c.heads, G = c.kv_heads, rep = H / G, GD = G * D, HD = H * D;
   const int KST = GD + 8;
   bf16_t* ks = reinterpret_cast<bf16_t*>(sa_lds);                       // [32][KST]
-  bf16_t* wm = ks + SA_KN * KST;                                         // [H][16][40] mixed weights
-  float* ps = reinterpret_cast<float*>(wm + (size_t)H * 16 * SA_WST);    // [H][16][33] weights
+  float* ps = reinterpret_cast<float*>(ks + SA_KN * KST);                // [H][16][33] weights (fp32) ...
+  bf16_t* wm = reinterpret_cast<bf16_t*>(ps);                            // ... and, once every wavefront has mixed, [H][16][40] bf16
   float* kis = ps + (size_t)H * 16 * SA_PST;                             // [32][G]
   float* tks = kis + SA_KN * G;                                          // [H][H]
   const int b = blockIdx.y, tile = gridDim.x - 1 - blockIdx.x;            // long rows first
@@ -689,23 +689,46 @@ __global__ void __launch_bounds__(256) sigattn_mfma_kernel(ktx_sigattn_config c,
   }
   // all heads of this wavefront on one key head?  (wave-uniform)
   const bool shared_kv = (h0 / rep) == ((min(h0 + NHW, H) - 1) / rep);
-  const int sj = tid >> 3, sx = (tid & 7) * 8;        // staging: 8 threads per key row, 16-byte pieces 64 elements apart
+  // staging: 8 threads per key row, 16-byte pieces 64 elements apart; a tile's rows are requested one tile ahead and wait in
+  // registers (SA_PF pieces of 16 bytes per thread cover key rows of up to 64 * SA_PF elements; longer rows are loaded in place)
+  constexpr int SA_PF = 8;
+  const int sj = tid >> 3, sx = (tid & 7) * 8;
+  uint4 pf[SA_PF];
+  float pf_ki = 0.f;
+  auto request = [&](int jt) {
+    const int j = jt * SA_KN + sj;
+    const bool ok = jt < jt1 && j <= p_last;
+    const size_t r = ok ? (size_t)pages[j / c.page_size] * c.page_size + (j % c.page_size) : 0;
+    const bf16_t* src = kcache + r * GD;
+#pragma unroll
+    for (int u = 0; u < SA_PF; u++) {
+      const int x = sx + u * 64;
+      pf[u] = (ok && x < GD) ? *reinterpret_cast<const uint4*>(src + x) : uint4{0u, 0u, 0u, 0u};
+    }
+    const int g = tid & 7;                 // thread g of a row's eight fetches 1 / rms of key head g (+8, +16 ... in place below)
+    pf_ki = (ok && g < G) ? kinv[r * G + g] : 0.f;
+  };
+  request(jt0);
   for (int jt = jt0; jt < jt1; jt++) {
     const int j0 = jt * SA_KN;
     __syncthreads();
     {
-      const int j = j0 + sj;
-      const bool ok = j <= p_last;
-      const size_t r = ok ? (size_t)pages[j / c.page_size] * c.page_size + (j % c.page_size) : 0;
-      const bf16_t* src = kcache + r * GD;
-      for (int x = sx; x < GD; x += 64) {
-        uint4 v = {0u, 0u, 0u, 0u};
-        if (ok) v = *reinterpret_cast<const uint4*>(src + x);
-        *reinterpret_cast<uint4*>(ks + sj * KST + x) = v;
+#pragma unroll
+      for (int u = 0; u < SA_PF; u++) {
+        const int x = sx + u * 64;
+        if (x < GD) *reinterpret_cast<uint4*>(ks + sj * KST + x) = pf[u];
       }
-      if ((tid & 7) == 0)
-        for (int g = 0; g < G; g++) kis[sj * G + g] = ok ? kinv[r * G + g] : 0.f;
+      if ((tid & 7) < G) kis[sj * G + (tid & 7)] = pf_ki;
+      if (GD > 64 * SA_PF || G > 8) {       // the part of wide rows the registers do not hold
+        const int j = j0 + sj;
+        const bool ok = j <= p_last;
+        const size_t r = ok ? (size_t)pages[j / c.page_size] * c.page_size + (j % c.page_size) : 0;
+        for (int x = sx + 64 * SA_PF; x < GD; x += 64)
+          *reinterpret_cast<uint4*>(ks + sj * KST + x) = ok ? *reinterpret_cast<const uint4*>(kcache + r * GD + x) : uint4{0u, 0u, 0u, 0u};
+        for (int g = 8 + (tid & 7); g < G; g += 8) kis[sj * G + g] = ok ? kinv[r * G + g] : 0.f;
+      }
     }
+    request(jt + 1);
     __syncthreads();
     // scores -> weights (fp32) of this wavefront's heads
 #pragma unroll
@@ -739,27 +762,44 @@ __global__ void __launch_bounds__(256) sigattn_mfma_kernel(ktx_sigattn_config c,
       }
     }
     __syncthreads();
-    // head mixing (fp32), then bf16 for the value product; rows of the tile that do not exist are skipped (decode steps have one)
-    if (lq * 4 < nrows) {
+    // head mixing (fp32) into registers; when every wavefront has read the fp32 tiles, the bf16 results take their place.
+    // A decode step's tile has one row: its wavefronts mix two weights per lane instead of eight.
+    {
       float wacc[NHW][8];
 #pragma unroll
       for (int u = 0; u < NHW; u++)
 #pragma unroll
         for (int x = 0; x < 8; x++) wacc[u][x] = 0.f;
-      for (int g = 0; g < H; g++) {
-        float pv[8];
+      if (nrows == 1) {
+        if (lq == 0) {
+          for (int g = 0; g < H; g++) {
+            const float pv0 = ps[(g * 16) * SA_PST + l16], pv1 = ps[(g * 16) * SA_PST + 16 + l16];
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++)
+            for (int u = 0; u < NHW; u++) {
+              const int h = h0 + u;
+              const float tk = h < H ? tks[h * H + g] : 0.f;
+              wacc[u][0] = fmaf(tk, pv0, wacc[u][0]);
+              wacc[u][4] = fmaf(tk, pv1, wacc[u][4]);
+            }
+          }
+        }
+      } else if (lq * 4 < nrows) {
+        for (int g = 0; g < H; g++) {
+          float pv[8];
 #pragma unroll
-          for (int r = 0; r < 4; r++) pv[nt * 4 + r] = ps[(g * 16 + lq * 4 + r) * SA_PST + nt * 16 + l16];
+          for (int nt = 0; nt < 2; nt++)
 #pragma unroll
-        for (int u = 0; u < NHW; u++) {
-          const int h = h0 + u;
-          const float tk = h < H ? tks[h * H + g] : 0.f;
+            for (int r = 0; r < 4; r++) pv[nt * 4 + r] = ps[(g * 16 + lq * 4 + r) * SA_PST + nt * 16 + l16];
 #pragma unroll
-          for (int x = 0; x < 8; x++) wacc[u][x] = fmaf(tk, pv[x], wacc[u][x]);
+          for (int u = 0; u < NHW; u++) {
+            const int h = h0 + u;
+            const float tk = h < H ? tks[h * H + g] : 0.f;
+#pragma unroll
+            for (int x = 0; x < 8; x++) wacc[u][x] = fmaf(tk, pv[x], wacc[u][x]);
+          }
         }
       }
+      __syncthreads();
 #pragma unroll
       for (int u = 0; u < NHW; u++) {
         const int h = h0 + u;
@@ -768,17 +808,6 @@ __global__ void __launch_bounds__(256) sigattn_mfma_kernel(ktx_sigattn_config c,
           for (int nt = 0; nt < 2; nt++)
 #pragma unroll
             for (int r = 0; r < 4; r++) wm[(h * 16 + lq * 4 + r) * SA_WST + nt * 16 + l16] = to_bf16_rne(wacc[u][nt * 4 + r]);
-        }
-      }
-    } else {
-#pragma unroll
-      for (int u = 0; u < NHW; u++) {
-        const int h = h0 + u;
-        if (h < H) {
-#pragma unroll
-          for (int nt = 0; nt < 2; nt++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) wm[(h * 16 + lq * 4 + r) * SA_WST + nt * 16 + l16] = 0;
         }
       }
     }
@@ -830,7 +859,7 @@ __global__ void __launch_bounds__(256) sigattn_mfma_kernel(ktx_sigattn_config c,
 
 size_t sigattn_mfma_lds(const ktx_sigattn_config& c) {
   const size_t GD = (size_t)c.kv_heads * c.dim, H = c.heads;
-  return SA_KN * (GD + 8) * 2 + H * 16 * SA_WST * 2 + H * 16 * SA_PST * 4 + SA_KN * c.kv_heads * 4 + H * H * 4;
+  return SA_KN * (GD + 8) * 2 + H * 16 * SA_PST * 4 + SA_KN * c.kv_heads * 4 + H * H * 4;      // (the bf16 tiles reuse the fp32 ones)
 }
 
 // ---------------------------------------------------------------------------------------------------------------------

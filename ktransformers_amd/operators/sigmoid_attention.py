@@ -69,7 +69,7 @@ class KSigmoidTalkAttention(BaseInjectedModule):
         if self.compute_dtype == torch.bfloat16 and sigattn_prefill_eligible(cfg):
             # matrix-core kernel: tiles of 16 query rows x key ranges, enough workgroups to fill the chip
             tiles = batch.B * ((batch.max_q_len + 15) // 16)
-            nsplit = max(1, min(self.TARGET_WORKGROUPS // max(tiles, 1), (batch.max_kv_len + 63) // 64))
+            nsplit = max(1, min(self.TARGET_WORKGROUPS // max(tiles, 1), (batch.max_kv_len + 31) // 32))
             a = sigattn_prefill(cfg, q, kc, kinv, batch.q_indptr, batch.pos0, batch.page_indptr, batch.page_indices, self.w["pb"],
                                 self.w["talk"], batch.max_q_len, nsplit=nsplit)
             return dense_gemm(a, self.w["o"])
