@@ -304,8 +304,17 @@ __global__ void __launch_bounds__(256) sigattn_reduce_kernel(int nsplit, size_t 
                                                              OT* __restrict__ out) {
   const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (e >= n) return;
+  // eight loads in flight per round; the sum stays in range order (a0 + a1 + ...), whatever nsplit is
   float a = 0.f;
-  for (int s = 0; s < nsplit; s++) a += partial[(size_t)s * n + e];
+  int s = 0;
+  for (; s + 8 <= nsplit; s += 8) {
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = partial[(size_t)(s + i) * n + e];
+#pragma unroll
+    for (int i = 0; i < 8; i++) a += v[i];
+  }
+  for (; s < nsplit; s++) a += partial[(size_t)s * n + e];
   st_elem(out, e, a);
 }
 
@@ -695,10 +704,17 @@ __global__ void __launch_bounds__(256) sigattn_mfma_kernel(ktx_sigattn_config c,
   const int sj = tid >> 3, sx = (tid & 7) * 8;
   uint4 pf[SA_PF];
   float pf_ki = 0.f;
-  auto request = [&](int jt) {
+  auto row_of = [&](int jt) -> long {      // cache row of this thread's key of tile jt, -1 when the key does not exist
     const int j = jt * SA_KN + sj;
-    const bool ok = jt < jt1 && j <= p_last;
-    const size_t r = ok ? (size_t)pages[j / c.page_size] * c.page_size + (j % c.page_size) : 0;
+    if (jt >= jt1 || j > p_last) return -1;
+    return (long)pages[j / c.page_size] * c.page_size + (j % c.page_size);
+  };
+  long row_next = row_of(jt0), row_cur = -1;    // the page lookup runs one tile ahead of the row loads, which run one tile ahead of use
+  auto request = [&](int jt) {
+    row_cur = row_next;
+    row_next = row_of(jt + 1);
+    const bool ok = row_cur >= 0;
+    const size_t r = ok ? (size_t)row_cur : 0;
     const bf16_t* src = kcache + r * GD;
 #pragma unroll
     for (int u = 0; u < SA_PF; u++) {
