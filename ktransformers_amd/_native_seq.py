@@ -50,7 +50,7 @@ def _load() -> C.CDLL:
     lib.ktx_sigattn_prefill.argtypes = [C.POINTER(_SigAttnConfig), C.c_int, C.c_int, C.c_int] + [C.c_void_p] * 9 + [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
     lib.ktx_gelu_tanh.argtypes = [C.c_size_t, C.c_void_p, C.c_int, C.c_void_p]
     lib.ktx_mlstm_forward.argtypes = [C.POINTER(_MlstmConfig), C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64] + [
-        C.c_int] * 5 + [C.c_void_p] * 8
+        C.c_int] * 5 + [C.c_void_p] * 7 + [C.c_int, C.c_void_p]
     lib.ktx_mlstm_gate_norm.argtypes = [C.POINTER(_MlstmConfig), C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p,
                                         C.c_void_p, C.c_int, C.c_void_p]
     lib.ktx_rms_combine.argtypes = [C.c_int, C.c_int] + [C.c_void_p] * 5 + [C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p,
@@ -200,7 +200,8 @@ def mlstm_config(heads: int, dim: int, vdim: int, gate_cap: float, eps: float, d
 
 
 def mlstm_forward(cfg: _MlstmConfig, proj: torch.Tensor, offs: dict, ib: torch.Tensor, fb: torch.Tensor, q_indptr: torch.Tensor,
-                  pos0: torch.Tensor, slot: torch.Tensor, S: torch.Tensor, n: torch.Tensor, m: torch.Tensor) -> torch.Tensor:
+                  pos0: torch.Tensor, slot: torch.Tensor, S: torch.Tensor, n: torch.Tensor, m: torch.Tensor,
+                  max_q_len: int | None = None) -> torch.Tensor:
     """The recurrence over the flattened batch (ktx_mlstm_forward); offs = column offsets of q, k, v, i, f in proj's rows.
     Returns the un-normed outputs fp32 [T, heads * vdim]; the state tensors are updated in place."""
     for t, what in ((q_indptr, "q_indptr"), (pos0, "pos0"), (slot, "slot")):
@@ -211,10 +212,11 @@ def mlstm_forward(cfg: _MlstmConfig, proj: torch.Tensor, offs: dict, ib: torch.T
         raise KtxError("mlstm_forward: proj must be fp32 rows")
     B, T = slot.numel(), proj.shape[0]
     o = torch.empty((T, cfg.heads * cfg.vdim), dtype=torch.float32, device=proj.device)
-    gates = torch.empty((T, cfg.heads, 3), dtype=torch.float32, device=proj.device)
+    gates = torch.empty(((B + 6 * T) * cfg.heads,), dtype=torch.float32, device=proj.device)
     check(lib.ktx_mlstm_forward(C.byref(cfg), B, q_indptr.data_ptr(), pos0.data_ptr(), slot.data_ptr(), proj.data_ptr(), proj.stride(0),
                                 offs["q"], offs["k"], offs["v"], offs["i"], offs["f"], ib.data_ptr(), fb.data_ptr(), S.data_ptr(),
-                                n.data_ptr(), m.data_ptr(), gates.data_ptr(), o.data_ptr(), _stream_ptr(proj.device)))
+                                n.data_ptr(), m.data_ptr(), gates.data_ptr(), o.data_ptr(), int(T if max_q_len is None else max_q_len),
+                                _stream_ptr(proj.device)))
     return o
 
 

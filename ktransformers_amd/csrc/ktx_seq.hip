@@ -322,12 +322,15 @@ __global__ void __launch_bounds__(256) sigattn_reduce_kernel(int nsplit, size_t 
 // mLSTM, part 1: the gates of a request's new tokens and the running maximum, off the sequential path.  Workgroup = (request, head).
 //   z_i, z_f -> log gates i_t, f_t (soft cap, logsigmoid);  m_t = max(f_t + m_(t-1), i_t) is a scan of maps m -> max(m + L, Z), which
 //   compose associatively ((L1, Z1) then (L2, Z2) = (L1 + L2, max(Z1 + L2, Z2))): 256 tokens per round, a wave scan on shuffles and
-//   the four wave totals through LDS.  Written per token: a_t = exp(f_t + m_(t-1) - m_t), b_t = exp(i_t - m_t), e_t = exp(-m_t).
+//   the four wave totals through LDS.  Written per token: a_t = exp(f_t + m_(t-1) - m_t), b_t = exp(i_t - m_t), e_t = exp(-m_t), and
+//   f_t, i_t, m_t themselves (the chunk kernel forms its own differences); per (request, head) the maximum the call started from.
+constexpr int KTX_MLSTM_GATE_FLOATS = 6;
 __global__ void __launch_bounds__(256) mlstm_gates_kernel(ktx_mlstm_config c, const int32_t* __restrict__ q_indptr,
                                                           const int32_t* __restrict__ pos0, const int32_t* __restrict__ slot,
                                                           const float* __restrict__ proj, int64_t ldp, int i_off, int f_off,
                                                           const float* __restrict__ ib, const float* __restrict__ fb,
-                                                          float* __restrict__ mg, float* __restrict__ gates) {
+                                                          float* __restrict__ mg, float* __restrict__ gates,
+                                                          float* __restrict__ minit) {
   __shared__ float wl[4], wz[4], mlast[256 + 1];
   __shared__ float m_carry;
   const int N = c.heads;
@@ -335,7 +338,10 @@ __global__ void __launch_bounds__(256) mlstm_gates_kernel(ktx_mlstm_config c, co
   const int t0 = q_indptr[b], t1 = q_indptr[b + 1];
   if (t1 <= t0) return;
   const int sl = slot[b];
-  if (tid == 0) m_carry = pos0[b] == 0 ? 0.f : mg[(size_t)sl * N + hd];
+  if (tid == 0) {
+    m_carry = pos0[b] == 0 ? 0.f : mg[(size_t)sl * N + hd];
+    minit[(size_t)b * N + hd] = m_carry;
+  }
   const float bi = ib[hd], bf = fb[hd], cap = c.gate_cap;
   for (int base = t0; base < t1; base += 256) {
     const int t = base + tid;
@@ -376,10 +382,13 @@ __global__ void __launch_bounds__(256) mlstm_gates_kernel(ktx_mlstm_config c, co
     __syncthreads();
     if (ok) {
       const float m_prev = mlast[tid];
-      float* g = gates + ((size_t)t * N + hd) * 3;
+      float* g = gates + ((size_t)t * N + hd) * KTX_MLSTM_GATE_FLOATS;
       g[0] = expf(lf + m_prev - m);
       g[1] = expf(zi - m);
       g[2] = expf(-m);
+      g[3] = lf;
+      g[4] = zi;
+      g[5] = m;
     }
     const int last = min(256, t1 - base) - 1;
     __syncthreads();
@@ -430,7 +439,7 @@ __global__ void __launch_bounds__(256) mlstm_fwd_kernel(ktx_mlstm_config c, cons
   float rq = 0.f, rk = 0.f, nv, na, nb, ne;
   {
     const float* row = proj + (size_t)t0 * ldp;
-    const float* g = gates + ((size_t)t0 * N + hd) * 3;
+    const float* g = gates + ((size_t)t0 * N + hd) * KTX_MLSTM_GATE_FLOATS;
     if (tid < D) {
       qk[0][0][tid] = row[q_off + hd * D + tid] * qscale;
       qk[0][1][tid] = row[k_off + hd * D + tid];
@@ -453,7 +462,7 @@ __global__ void __launch_bounds__(256) mlstm_fwd_kernel(ktx_mlstm_config c, cons
     }
     if (t + 1 < t1) {
       const float* row = proj + (size_t)(t + 1) * ldp;
-      const float* g = gates + ((size_t)(t + 1) * N + hd) * 3;
+      const float* g = gates + ((size_t)(t + 1) * N + hd) * KTX_MLSTM_GATE_FLOATS;
       nv = vok ? row[v_off + hd * V + v] : 0.f;
       na = g[0], nb = g[1], ne = g[2];
       if (t + 2 < t1 && tid < D) {
@@ -491,6 +500,171 @@ __global__ void __launch_bounds__(256) mlstm_fwd_kernel(ktx_mlstm_config c, cons
       if (vs == 0 && lane == 0) np_[d] = nn[i];
     }
   }
+}
+
+// mLSTM, part 2 for prompts: the same recurrence 16 tokens at a time on the matrix cores (fp32 MFMA: state, gates and products stay
+// fp32).  With F_t the sum of the chunk's log forget gates up to t and m_0 the maximum the chunk starts from, unrolling the recurrence
+// over a chunk gives
+//   S_t^T q_t = exp(F_t + m_0 - m_t) S_0^T q_t + sum_{s <= t} exp(F_t - F_s + i_s - m_t) (k_s . q_t) v_s        (n_t . q_t alike, without v)
+//   S_L       = exp(F_L + m_0 - m_L) S_0 + sum_s exp(F_L - F_s + i_s - m_L) k_s v_s^T
+// — every exponent is <= 0 because m is the running maximum of exactly these sums.  Workgroup = (request, head, 64 value columns), the
+// state slice [dim, 64] lives in LDS for the whole call; wavefront w owns 16 columns: A = Q K^T (16 x 16), W = A o weights (lower
+// triangle), O = c o (Q S_0) + W V, then its columns of S_L = decay S_0 + (u o K)^T V.  Only the staging of a chunk is shared.
+constexpr int ML_CL = 16;
+__global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, const int32_t* __restrict__ q_indptr,
+                                                          const int32_t* __restrict__ pos0, const int32_t* __restrict__ slot,
+                                                          const float* __restrict__ proj, int64_t ldp, int q_off, int k_off,
+                                                          int v_off, const float* __restrict__ gates, const float* __restrict__ minit,
+                                                          float* __restrict__ Sg, float* __restrict__ ng, float* __restrict__ o_raw) {
+  extern __shared__ __attribute__((aligned(16))) float cl[];
+  const int N = c.heads, D = c.dim, V = c.vdim;
+  const int Dp = (D + 15) & ~15, QST = Dp + 4;
+  float* Ss = cl;                           // [Dp][64]
+  float* Qs = Ss + (size_t)Dp * 64;         // [16][QST]
+  float* Ks = Qs + ML_CL * QST;             // [16][QST]
+  float* Vs = Ks + ML_CL * QST;             // [16][64]
+  float* Ws = Vs + ML_CL * 64;              // [4][16][17]
+  float* ns = Ws + 4 * 16 * 17;             // [2][Dp]
+  float* gl = ns + 2 * Dp;                  // lf[16] zi[16] m[16] | rt[16] ct[16] cc[16] ee[16] us[16] | decay, m_last
+  float* qn = gl + 8 * 16 + 2;              // [4][16]
+  const int b = blockIdx.x, hd = blockIdx.y, vs = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int t0 = q_indptr[b], t1 = q_indptr[b + 1];
+  if (t1 <= t0) return;
+  const int sl = slot[b];
+  const bool fresh = pos0[b] == 0;
+  float* Sp = Sg + ((size_t)sl * N + hd) * D * V;
+  float* np_ = ng + ((size_t)sl * N + hd) * D;
+  for (int e = tid; e < Dp * 64; e += 256) {
+    const int d = e >> 6, col = e & 63, v = vs * 64 + col;
+    Ss[e] = (!fresh && d < D && v < V) ? Sp[(size_t)d * V + v] : 0.f;
+  }
+  for (int d = tid; d < Dp; d += 256) ns[d] = (!fresh && d < D) ? np_[d] : 0.f;
+  float m0 = minit[(size_t)b * N + hd];
+  const float qscale = 1.0f / sqrtf((float)D);
+  const int vcol = 16 * wave + l16, v = vs * 64 + vcol;
+  const bool vok = v < V;
+  float* Ww = Ws + wave * 16 * 17;
+  float* qnw = qn + wave * 16;
+  int par = 0;
+  for (int c0 = t0; c0 < t1; c0 += ML_CL, par ^= 1) {
+    const int nv = min(ML_CL, t1 - c0);
+    float* n_cur = ns + par * Dp;
+    float* n_nxt = ns + (par ^ 1) * Dp;
+    __syncthreads();
+    for (int e = tid; e < ML_CL * Dp; e += 256) {
+      const int t = e / Dp, d = e - t * Dp;
+      float qv = 0.f, kv = 0.f;
+      if (t < nv && d < D) {
+        const float* row = proj + (size_t)(c0 + t) * ldp;
+        qv = row[q_off + hd * D + d] * qscale;
+        kv = row[k_off + hd * D + d];
+      }
+      Qs[t * QST + d] = qv;
+      Ks[t * QST + d] = kv;
+    }
+    for (int e = tid; e < ML_CL * 64; e += 256) {
+      const int t = e >> 6, col = e & 63, vv = vs * 64 + col;
+      Vs[e] = (t < nv && vv < V) ? proj[(size_t)(c0 + t) * ldp + v_off + hd * V + vv] : 0.f;
+    }
+    if (tid < ML_CL) {
+      const float* g = gates + ((size_t)(c0 + min(tid, nv - 1)) * N + hd) * KTX_MLSTM_GATE_FLOATS;
+      gl[tid] = tid < nv ? g[3] : 0.f;
+      gl[16 + tid] = g[4];
+      gl[32 + tid] = g[5];
+    }
+    __syncthreads();
+    if (tid < ML_CL) {
+      float F = 0.f, FL = 0.f;
+      for (int r = 0; r < nv; r++) {
+        FL += gl[r];
+        if (r <= tid) F = FL;
+      }
+      const float mt = gl[32 + tid], zi = gl[16 + tid], mL = gl[32 + nv - 1];
+      const bool ok = tid < nv;
+      gl[48 + tid] = F - mt;                                   // row term of the weights
+      gl[64 + tid] = F - zi;                                   // column term
+      gl[80 + tid] = ok ? expf(F + m0 - mt) : 0.f;             // carry of the incoming state into token t
+      gl[96 + tid] = expf(-mt);
+      gl[112 + tid] = ok ? expf(FL - F + zi - mL) : 0.f;       // weight of token s in the outgoing state
+      if (tid == 0) {
+        gl[128] = expf(FL + m0 - mL);
+        gl[129] = mL;
+      }
+    }
+    __syncthreads();
+    const float decay = gl[128];
+    // (i) A = Q K^T, (ii) weights, row sums, relayout through the wavefront's LDS tile
+    v4f A = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < Dp; k += 4) A = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[l16 * QST + k + lq], Ks[l16 * QST + k + lq], A, 0, 0, 0);
+    float rsum[4];
+    {
+      const float ctm = gl[64 + l16];
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int t = lq * 4 + r;
+        float w = 0.f;
+        if (l16 <= t && t < nv) w = A[r] * expf(gl[48 + t] - ctm);
+        Ww[t * 17 + l16] = w;
+        rsum[r] = w;
+      }
+      row16_sum4(rsum[0], rsum[1], rsum[2], rsum[3]);
+    }
+    // (iii) q_t . n_0 for the 16 tokens
+    {
+      float pq = 0.f;
+      for (int k = lq; k < Dp; k += 4) pq += Qs[l16 * QST + k] * n_cur[k];
+      pq += __shfl_xor(pq, 16, 64);
+      pq += __shfl_xor(pq, 32, 64);
+      if (lq == 0) qnw[l16] = pq;
+    }
+    // (iv) O = carry o (Q S_0) + W V  -> outputs
+    v4f O = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < Dp; k += 4) O = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[l16 * QST + k + lq], Ss[(k + lq) * 64 + vcol], O, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 4; r++) O[r] *= gl[80 + lq * 4 + r];
+#pragma unroll
+    for (int k = 0; k < ML_CL; k += 4) O = __builtin_amdgcn_mfma_f32_16x16x4f32(Ww[l16 * 17 + k + lq], Vs[(k + lq) * 64 + vcol], O, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int t = lq * 4 + r;
+      if (t < nv && vok) {
+        const float nq = gl[80 + t] * qnw[t] + rsum[r];
+        o_raw[(size_t)(c0 + t) * N * V + hd * V + v] = O[r] / (fmaxf(fabsf(nq), gl[96 + t]) + c.denom_eps);
+      }
+    }
+    // (v) this wavefront's 16 columns of the outgoing state
+    for (int dt = 0; dt < Dp; dt += 16) {
+      v4f C;
+#pragma unroll
+      for (int r = 0; r < 4; r++) C[r] = decay * Ss[(dt + lq * 4 + r) * 64 + vcol];
+#pragma unroll
+      for (int k = 0; k < ML_CL; k += 4)
+        C = __builtin_amdgcn_mfma_f32_16x16x4f32(Ks[(k + lq) * QST + dt + l16] * gl[112 + k + lq], Vs[(k + lq) * 64 + vcol], C, 0, 0, 0);
+#pragma unroll
+      for (int r = 0; r < 4; r++) Ss[(dt + lq * 4 + r) * 64 + vcol] = C[r];
+    }
+    // (vi) the normaliser (into the other half: every wavefront may still be reading this chunk's)
+    for (int d = tid; d < Dp; d += 256) {
+      float a = decay * n_cur[d];
+      for (int s2 = 0; s2 < nv; s2++) a += gl[112 + s2] * Ks[s2 * QST + d];
+      n_nxt[d] = a;
+    }
+    m0 = gl[129];
+  }
+  __syncthreads();
+  for (int e = tid; e < Dp * 64; e += 256) {
+    const int d = e >> 6, col = e & 63, vv = vs * 64 + col;
+    if (d < D && vv < V) Sp[(size_t)d * V + vv] = Ss[e];
+  }
+  if (vs == 0)
+    for (int d = tid; d < D; d += 256) np_[d] = ns[par * Dp + d];
+}
+
+size_t mlstm_chunk_lds(int D) {
+  const size_t Dp = (D + 15) & ~15;
+  return (Dp * 64 + 2 * ML_CL * (Dp + 4) + ML_CL * 64 + 4 * 16 * 17 + 2 * Dp + 8 * 16 + 2 + 4 * 16) * sizeof(float);
 }
 
 template <typename OT>
@@ -1222,7 +1396,8 @@ int ktx_gelu_tanh(size_t n, void* d_y, int dtype, ktx_stream_t stream) {
 
 int ktx_mlstm_forward(const ktx_mlstm_config* cfg, int B, const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_slot,
                       const float* d_proj, int64_t ldp, int q_off, int k_off, int v_off, int i_off, int f_off, const float* d_ib,
-                      const float* d_fb, float* d_S, float* d_n, float* d_m, float* d_gates, float* d_o_raw, ktx_stream_t stream) {
+                      const float* d_fb, float* d_S, float* d_n, float* d_m, float* d_gates, float* d_o_raw, int max_q_len,
+                      ktx_stream_t stream) {
   KTX_REQUIRE(cfg && cfg->heads > 0 && cfg->dim > 0 && cfg->vdim > 0, "ktx_mlstm_forward: heads, dim, vdim must be positive");
   KTX_REQUIRE(cfg->dim <= 256, "ktx_mlstm_forward: dim must be <= 256 (a wavefront keeps dim / 4 state rows in registers)");
   KTX_REQUIRE(B >= 0 && d_q_indptr && d_pos0 && d_slot && d_proj && d_ib && d_fb && d_S && d_n && d_m && d_gates && d_o_raw,
@@ -1235,8 +1410,19 @@ int ktx_mlstm_forward(const ktx_mlstm_config* cfg, int B, const int32_t* d_q_ind
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid(B, cfg->heads, (cfg->vdim + 63) / 64);
   KTX_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "ktx_mlstm_forward: too many heads / value columns");
+  // scratch layout: [T][heads][6] gate records, then [B][heads] starting maxima; T is not known here, so the maxima come FIRST
+  float* minit = d_gates;
+  float* grec = d_gates + (size_t)B * cfg->heads;
   mlstm_gates_kernel<<<dim3(B, cfg->heads), 256, 0, st>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_proj, ldp, i_off, f_off, d_ib, d_fb, d_m,
-                                                          d_gates);
+                                                          grec, minit);
+  if (max_q_len >= ML_CL && mlstm_chunk_lds(cfg->dim) <= 150 * 1024) {
+    KTX_HIP(ktx_set_max_lds((const void*)mlstm_chunk_kernel, 160 * 1024));
+    mlstm_chunk_kernel<<<grid, 256, mlstm_chunk_lds(cfg->dim), st>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_proj, ldp, q_off, k_off, v_off,
+                                                                     grec, minit, d_S, d_n, d_o_raw);
+    KTX_HIP(hipGetLastError());
+    return 0;
+  }
+  d_gates = grec;
   const int dpg = (cfg->dim + 3) / 4;
 #define KTX_ML_GO(DPG)                                                                                                       \
   mlstm_fwd_kernel<DPG><<<grid, 256, 0, st>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_proj, ldp, q_off, k_off, v_off, d_gates, d_S, \

@@ -58,6 +58,6 @@ class KMLSTMMixer(BaseInjectedModule):
             c += rows
         li = self.layer_idx
         o_raw = mlstm_forward(self._cfg, proj, offs, self.w["i.b"], self.w["f.b"], batch.q_indptr, batch.pos0, batch.slot,
-                              cache.S[li], cache.n[li], cache.m[li])
+                              cache.S[li], cache.n[li], cache.m[li], max_q_len=batch.max_q_len)
         o = mlstm_gate_norm(self._cfg, o_raw, proj, offs["g"], self.w["norm"], self.compute_dtype)
         return dense_gemm(o, self.w["o"])

@@ -158,7 +158,7 @@ def test_sigmoid_attention_whole_and_portions(dtype, H, G, D):
     assert rel(_run_attention(c, P, h, dtype, [45], page_size=64), ref) < tol
 
 
-@pytest.mark.parametrize("H,G,D,T", [(4, 2, 32, 45), (8, 8, 96, 130), (6, 3, 64, 33), (16, 4, 128, 70), (1, 1, 32, 17), (13, 1, 64, 40)])
+@pytest.mark.parametrize("H,G,D,T", [(4, 2, 32, 45), (4, 4, 96, 130), (6, 3, 64, 33), (16, 4, 128, 70), (1, 1, 32, 17), (13, 1, 64, 40)])
 def test_sigmoid_attention_matrix_core_kernel(H, G, D, T):
     """The prompt kernel (16-row tiles x all heads, bf16 MFMA) against the plain statement: whole prompts, portions that start in the
     middle of a tile and of a page, several requests of unequal length in one call."""
@@ -241,7 +241,7 @@ def _mlstm_case(seed, N, D, V, T, width=24, cap=6.0):
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
-@pytest.mark.parametrize("N,D,V", [(2, 8, 16), (1, 5, 7), (3, 48, 64), (1, 24, 80), (2, 130, 33)])
+@pytest.mark.parametrize("N,D,V", [(2, 8, 16), (1, 5, 7), (3, 40, 72), (1, 24, 80), (2, 130, 33)])
 def test_mlstm_whole_portions_and_state_carry(dtype, N, D, V):
     from ktransformers_amd._native_seq import dense_gemm, mlstm_config, mlstm_forward, mlstm_gate_norm
     from ktransformers_amd.models.custom_cache import KHybridCache
