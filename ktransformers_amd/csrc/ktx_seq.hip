@@ -547,33 +547,57 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, co
   const bool vok = v < V;
   float* Ww = Ws + wave * 16 * 17;
   float* qnw = qn + wave * 16;
+  // a chunk's q / k / v / gate records are requested one chunk ahead and wait in registers
+  constexpr int ML_PF = 16;                   // 256 threads x 16 cover the 16 x Dp (Dp <= 256) elements of q and of k
+  float rq[ML_PF], rk[ML_PF], rv[4], rg[3] = {0.f, 0.f, 0.f};
+  auto fetch = [&](int c0) {
+    const int nv = min(ML_CL, t1 - c0);
+#pragma unroll
+    for (int i = 0; i < ML_PF; i++) {
+      const int e = tid + i * 256;
+      const int t = e / Dp, d = e - t * Dp;
+      const bool ok = e < ML_CL * Dp && t < nv && d < D;
+      const float* row = proj + (size_t)(c0 + (ok ? t : 0)) * ldp;
+      rq[i] = ok ? row[q_off + hd * D + d] : 0.f;
+      rk[i] = ok ? row[k_off + hd * D + d] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int e = tid + i * 256;
+      const int t = e >> 6, vv = vs * 64 + (e & 63);
+      rv[i] = (t < nv && vv < V) ? proj[(size_t)(c0 + t) * ldp + v_off + hd * V + vv] : 0.f;
+    }
+    if (tid < ML_CL && nv > 0) {
+      const float* g = gates + ((size_t)(c0 + min(tid, nv - 1)) * N + hd) * KTX_MLSTM_GATE_FLOATS;
+      rg[0] = tid < nv ? g[3] : 0.f;
+      rg[1] = g[4];
+      rg[2] = g[5];
+    }
+  };
+  fetch(t0);
   int par = 0;
   for (int c0 = t0; c0 < t1; c0 += ML_CL, par ^= 1) {
     const int nv = min(ML_CL, t1 - c0);
     float* n_cur = ns + par * Dp;
     float* n_nxt = ns + (par ^ 1) * Dp;
     __syncthreads();
-    for (int e = tid; e < ML_CL * Dp; e += 256) {
-      const int t = e / Dp, d = e - t * Dp;
-      float qv = 0.f, kv = 0.f;
-      if (t < nv && d < D) {
-        const float* row = proj + (size_t)(c0 + t) * ldp;
-        qv = row[q_off + hd * D + d] * qscale;
-        kv = row[k_off + hd * D + d];
+#pragma unroll
+    for (int i = 0; i < ML_PF; i++) {
+      const int e = tid + i * 256;
+      if (e < ML_CL * Dp) {
+        const int t = e / Dp, d = e - t * Dp;
+        Qs[t * QST + d] = rq[i] * qscale;
+        Ks[t * QST + d] = rk[i];
       }
-      Qs[t * QST + d] = qv;
-      Ks[t * QST + d] = kv;
     }
-    for (int e = tid; e < ML_CL * 64; e += 256) {
-      const int t = e >> 6, col = e & 63, vv = vs * 64 + col;
-      Vs[e] = (t < nv && vv < V) ? proj[(size_t)(c0 + t) * ldp + v_off + hd * V + vv] : 0.f;
-    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) Vs[tid + i * 256] = rv[i];
     if (tid < ML_CL) {
-      const float* g = gates + ((size_t)(c0 + min(tid, nv - 1)) * N + hd) * KTX_MLSTM_GATE_FLOATS;
-      gl[tid] = tid < nv ? g[3] : 0.f;
-      gl[16 + tid] = g[4];
-      gl[32 + tid] = g[5];
+      gl[tid] = rg[0];
+      gl[16 + tid] = rg[1];
+      gl[32 + tid] = rg[2];
     }
+    if (c0 + ML_CL < t1) fetch(c0 + ML_CL);
     __syncthreads();
     if (tid < ML_CL) {
       float F = 0.f, FL = 0.f;
@@ -597,6 +621,7 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, co
     const float decay = gl[128];
     // (i) A = Q K^T, (ii) weights, row sums, relayout through the wavefront's LDS tile
     v4f A = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
     for (int k = 0; k < Dp; k += 4) A = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[l16 * QST + k + lq], Ks[l16 * QST + k + lq], A, 0, 0, 0);
     float rsum[4];
     {
@@ -614,6 +639,7 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, co
     // (iii) q_t . n_0 for the 16 tokens
     {
       float pq = 0.f;
+#pragma unroll 8
       for (int k = lq; k < Dp; k += 4) pq += Qs[l16 * QST + k] * n_cur[k];
       pq += __shfl_xor(pq, 16, 64);
       pq += __shfl_xor(pq, 32, 64);
@@ -621,6 +647,7 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, co
     }
     // (iv) O = carry o (Q S_0) + W V  -> outputs
     v4f O = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
     for (int k = 0; k < Dp; k += 4) O = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[l16 * QST + k + lq], Ss[(k + lq) * 64 + vcol], O, 0, 0, 0);
 #pragma unroll
     for (int r = 0; r < 4; r++) O[r] *= gl[80 + lq * 4 + r];
@@ -635,6 +662,7 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, co
       }
     }
     // (v) this wavefront's 16 columns of the outgoing state
+#pragma unroll 2
     for (int dt = 0; dt < Dp; dt += 16) {
       v4f C;
 #pragma unroll
