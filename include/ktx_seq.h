@@ -37,7 +37,7 @@ int ktx_embed_sinpos(int T, int width, int vocab, const int32_t* d_tokens, const
 int ktx_dense_gemm(int M, int N, int K, const void* d_A, int a_dtype, int64_t lda, const void* d_W, int w_dtype, void* d_Y,
                    int y_dtype, int64_t ldy, int act, int ksplit, ktx_stream_t stream);
 
-typedef struct {
+typedef struct ktx_sigattn_config {
   int32_t heads, kv_heads, dim;   /* query heads, key heads (heads % kv_heads == 0), per-head size of q, k and v (v = k) */
   float scale;                    /* score = scale * (q . k) */
   float temp_coef;                /* q *= 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1); 0 switches it off */
@@ -79,7 +79,7 @@ int ktx_sigattn_prefill(const ktx_sigattn_config* cfg, int B, int T, int max_q_l
 /* y = gelu_tanh(y) in place, n elements of `dtype` (the activation behind a GEMM that has no epilogue for it). */
 int ktx_gelu_tanh(size_t n, void* d_y, int dtype, ktx_stream_t stream);
 
-typedef struct {
+typedef struct ktx_mlstm_config {
   int32_t heads, dim, vdim;       /* per head: q, k of size dim, v of size vdim; state S [dim][vdim], n [dim], m */
   float gate_cap;                 /* log gates are soft-capped: cap * tanh(z / cap); 0 = no cap */
   float eps;                      /* of the per-head unit norm on the output */

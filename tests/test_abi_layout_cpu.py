@@ -12,7 +12,9 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PAIRS = [("ktx_moe_config", "_MoeConfig", "ktx_moe.h"), ("ktx_linear_config", "_LinearConfig", "ktx_linear.h"),
          ("ktx_linear_fusion", "_LinearFusion", "ktx_linear.h"), ("ktx_gate_config", "_GateConfig", "ktx_gate.h"),
          ("ktx_mla_config", "_MlaConfig", "ktx_mla.h"), ("ktx_gemm_args", "_GemmArgs", "ktx_gemm.h"),
-         ("ktx_attn_decode_args", "_AttnDecodeArgs", "ktx_attn.h")]
+         ("ktx_attn_decode_args", "_AttnDecodeArgs", "ktx_attn.h"),
+         # (the sequence-mixer structs are mirrored in ktransformers_amd/_native_seq.py)
+         ("ktx_sigattn_config", "_SigAttnConfig", "ktx_seq.h"), ("ktx_mlstm_config", "_MlstmConfig", "ktx_seq.h")]
 
 
 @pytest.fixture(scope="module")
@@ -21,7 +23,12 @@ def native():
         from ktransformers_amd import _native
     except ImportError as e:          # the library is built by __graft_entry__.build(); without it there is nothing to mirror
         pytest.skip(f"libktx_hip.so not built: {e}")
-    return _native
+    from ktransformers_amd import _native_seq
+
+    class Both:
+        def __getattr__(self, name):
+            return getattr(_native, name) if hasattr(_native, name) else getattr(_native_seq, name)
+    return Both()
 
 
 def test_ctypes_mirrors_match_the_headers(native, tmp_path):
