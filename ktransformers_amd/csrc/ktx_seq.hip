@@ -621,8 +621,20 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, co
     const float decay = gl[128];
     // (i) A = Q K^T, (ii) weights, row sums, relayout through the wavefront's LDS tile
     v4f A = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 8
-    for (int k = 0; k < Dp; k += 4) A = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[l16 * QST + k + lq], Ks[l16 * QST + k + lq], A, 0, 0, 0);
+    {
+      // four independent accumulators (Dp is a multiple of 16): the products of one chain wait on each other otherwise
+      v4f a1 = A, a2 = A, a3 = A;
+      const float* qr = Qs + l16 * QST + lq;
+      const float* kr = Ks + l16 * QST + lq;
+#pragma unroll 2
+      for (int k = 0; k < Dp; k += 16) {
+        A = __builtin_amdgcn_mfma_f32_16x16x4f32(qr[k], kr[k], A, 0, 0, 0);
+        a1 = __builtin_amdgcn_mfma_f32_16x16x4f32(qr[k + 4], kr[k + 4], a1, 0, 0, 0);
+        a2 = __builtin_amdgcn_mfma_f32_16x16x4f32(qr[k + 8], kr[k + 8], a2, 0, 0, 0);
+        a3 = __builtin_amdgcn_mfma_f32_16x16x4f32(qr[k + 12], kr[k + 12], a3, 0, 0, 0);
+      }
+      A = (A + a1) + (a2 + a3);
+    }
     float rsum[4];
     {
       const float ctm = gl[64 + l16];
@@ -647,8 +659,19 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, co
     }
     // (iv) O = carry o (Q S_0) + W V  -> outputs
     v4f O = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 8
-    for (int k = 0; k < Dp; k += 4) O = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[l16 * QST + k + lq], Ss[(k + lq) * 64 + vcol], O, 0, 0, 0);
+    {
+      v4f o1 = O, o2 = O, o3 = O;
+      const float* qr = Qs + l16 * QST + lq;
+      const float* sr = Ss + lq * 64 + vcol;
+#pragma unroll 2
+      for (int k = 0; k < Dp; k += 16) {
+        O = __builtin_amdgcn_mfma_f32_16x16x4f32(qr[k], sr[k * 64], O, 0, 0, 0);
+        o1 = __builtin_amdgcn_mfma_f32_16x16x4f32(qr[k + 4], sr[(k + 4) * 64], o1, 0, 0, 0);
+        o2 = __builtin_amdgcn_mfma_f32_16x16x4f32(qr[k + 8], sr[(k + 8) * 64], o2, 0, 0, 0);
+        o3 = __builtin_amdgcn_mfma_f32_16x16x4f32(qr[k + 12], sr[(k + 12) * 64], o3, 0, 0, 0);
+      }
+      O = (O + o1) + (o2 + o3);
+    }
 #pragma unroll
     for (int r = 0; r < 4; r++) O[r] *= gl[80 + lq * 4 + r];
 #pragma unroll
