@@ -93,7 +93,7 @@ typedef struct ktx_mlstm_config {
  *   S' = exp(f + m - m') S + exp(i - m') k v^T, n' likewise with k, o = S'^T q / (max(|n' . q|, exp(-m')) + denom_eps).
  * S: fp32 [slots][heads][dim][vdim], n: [slots][heads][dim], m: [slots][heads].  o_raw: fp32 [T][heads*vdim].
  * Two launches: the gates and the running maximum of all new tokens (a scan, off the sequential path) into d_gates, fp32 scratch of
- * (B + 6 T) * heads floats, then the state recurrence — token by token, or, when the longest request brings max_q_len >= 16 tokens,
+ * (B + 8 T) * heads floats, then the state recurrence — token by token, or, when the longest request brings max_q_len >= 16 tokens,
  * 16 tokens at a time on the fp32 matrix cores (the recurrence unrolled over a chunk; same numbers up to fp32 rounding). */
 int ktx_mlstm_forward(const ktx_mlstm_config* cfg, int B, const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_slot,
                       const float* d_proj, int64_t ldp, int q_off, int k_off, int v_off, int i_off, int f_off, const float* d_ib,

@@ -212,7 +212,7 @@ def mlstm_forward(cfg: _MlstmConfig, proj: torch.Tensor, offs: dict, ib: torch.T
         raise KtxError("mlstm_forward: proj must be fp32 rows")
     B, T = slot.numel(), proj.shape[0]
     o = torch.empty((T, cfg.heads * cfg.vdim), dtype=torch.float32, device=proj.device)
-    gates = torch.empty(((B + 6 * T) * cfg.heads,), dtype=torch.float32, device=proj.device)
+    gates = torch.empty(((B + 8 * T) * cfg.heads,), dtype=torch.float32, device=proj.device)
     check(lib.ktx_mlstm_forward(C.byref(cfg), B, q_indptr.data_ptr(), pos0.data_ptr(), slot.data_ptr(), proj.data_ptr(), proj.stride(0),
                                 offs["q"], offs["k"], offs["v"], offs["i"], offs["f"], ib.data_ptr(), fb.data_ptr(), S.data_ptr(),
                                 n.data_ptr(), m.data_ptr(), gates.data_ptr(), o.data_ptr(), int(T if max_q_len is None else max_q_len),

@@ -323,15 +323,15 @@ __global__ void __launch_bounds__(256) sigattn_reduce_kernel(int nsplit, size_t 
 //   z_i, z_f -> log gates i_t, f_t (soft cap, logsigmoid);  m_t = max(f_t + m_(t-1), i_t) is a scan of maps m -> max(m + L, Z), which
 //   compose associatively ((L1, Z1) then (L2, Z2) = (L1 + L2, max(Z1 + L2, Z2))): 256 tokens per round, a wave scan on shuffles and
 //   the four wave totals through LDS.  Written per token: a_t = exp(f_t + m_(t-1) - m_t), b_t = exp(i_t - m_t), e_t = exp(-m_t), and
-//   f_t, i_t, m_t themselves (the chunk kernel forms its own differences); per (request, head) the maximum the call started from.
-constexpr int KTX_MLSTM_GATE_FLOATS = 6;
+//   the five terms the chunk kernel multiplies with; per (request, head) the maximum the call started from.
+constexpr int KTX_MLSTM_GATE_FLOATS = 8;
 __global__ void __launch_bounds__(256) mlstm_gates_kernel(ktx_mlstm_config c, const int32_t* __restrict__ q_indptr,
                                                           const int32_t* __restrict__ pos0, const int32_t* __restrict__ slot,
                                                           const float* __restrict__ proj, int64_t ldp, int i_off, int f_off,
                                                           const float* __restrict__ ib, const float* __restrict__ fb,
                                                           float* __restrict__ mg, float* __restrict__ gates,
                                                           float* __restrict__ minit) {
-  __shared__ float wl[4], wz[4], mlast[256 + 1];
+  __shared__ float wl[4], wz[4], mlast[256 + 1], lfs[256];
   __shared__ float m_carry;
   const int N = c.heads;
   const int b = blockIdx.x, hd = blockIdx.y, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -386,9 +386,25 @@ __global__ void __launch_bounds__(256) mlstm_gates_kernel(ktx_mlstm_config c, co
       g[0] = expf(lf + m_prev - m);
       g[1] = expf(zi - m);
       g[2] = expf(-m);
-      g[3] = lf;
-      g[4] = zi;
-      g[5] = m;
+    }
+    // the terms of the 16-token chunk form (chunks are counted from the request's first new token; a round holds 16 whole chunks):
+    // F = the chunk's summed log forget gates up to the token, m_0 = the maximum before the chunk, L = the chunk's last token
+    lfs[tid] = ok ? lf : 0.f;
+    __syncthreads();
+    if (ok) {
+      const int cb = tid & ~15, nvc = min(16, t1 - (base + cb));
+      float F = 0.f, FL = 0.f;
+      for (int r = 0; r < nvc; r++) {
+        FL += lfs[cb + r];
+        if (cb + r <= tid) F = FL;
+      }
+      const float m0c = mlast[cb], mL = mlast[cb + nvc];
+      float* g = gates + ((size_t)t * N + hd) * KTX_MLSTM_GATE_FLOATS;
+      g[3] = F - m;                          // row term of the in-chunk weights exp(F_t - F_s + i_s - m_t)
+      g[4] = F - zi;                         // column term
+      g[5] = expf(F + m0c - m);              // carry of the chunk's incoming state into this token
+      g[6] = expf(FL - F + zi - mL);         // weight of this token in the chunk's outgoing state
+      g[7] = expf(FL + m0c - mL);            // decay of the incoming state over the whole chunk
     }
     const int last = min(256, t1 - base) - 1;
     __syncthreads();
@@ -525,7 +541,7 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, co
   float* Vs = Ks + ML_CL * QST;             // [16][64]
   float* Ws = Vs + ML_CL * 64;              // [4][16][17]
   float* ns = Ws + 4 * 16 * 17;             // [2][Dp]
-  float* gl = ns + 2 * Dp;                  // lf[16] zi[16] m[16] | rt[16] ct[16] cc[16] ee[16] us[16] | decay, m_last
+  float* gl = ns + 2 * Dp;                  // (48 unused) | rt[16] ct[16] cc[16] ee[16] us[16] | decay
   float* qn = gl + 8 * 16 + 2;              // [4][16]
   const int b = blockIdx.x, hd = blockIdx.y, vs = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
@@ -541,7 +557,6 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, co
     Ss[e] = (!fresh && d < D && v < V) ? Sp[(size_t)d * V + v] : 0.f;
   }
   for (int d = tid; d < Dp; d += 256) ns[d] = (!fresh && d < D) ? np_[d] : 0.f;
-  float m0 = minit[(size_t)b * N + hd];
   const float qscale = 1.0f / sqrtf((float)D);
   const int vcol = 16 * wave + l16, v = vs * 64 + vcol;
   const bool vok = v < V;
@@ -549,7 +564,7 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, co
   float* qnw = qn + wave * 16;
   // a chunk's q / k / v / gate records are requested one chunk ahead and wait in registers
   constexpr int ML_PF = 16;                   // 256 threads x 16 cover the 16 x Dp (Dp <= 256) elements of q and of k
-  float rq[ML_PF], rk[ML_PF], rv[4], rg[3] = {0.f, 0.f, 0.f};
+  float rq[ML_PF], rk[ML_PF], rv[4], rg[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   auto fetch = [&](int c0) {
     const int nv = min(ML_CL, t1 - c0);
 #pragma unroll
@@ -567,11 +582,15 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, co
       const int t = e >> 6, vv = vs * 64 + (e & 63);
       rv[i] = (t < nv && vv < V) ? proj[(size_t)(c0 + t) * ldp + v_off + hd * V + vv] : 0.f;
     }
-    if (tid < ML_CL && nv > 0) {
-      const float* g = gates + ((size_t)(c0 + min(tid, nv - 1)) * N + hd) * KTX_MLSTM_GATE_FLOATS;
-      rg[0] = tid < nv ? g[3] : 0.f;
-      rg[1] = g[4];
-      rg[2] = g[5];
+    if (tid < ML_CL) {
+      const bool okt = tid < nv;
+      const float* g = gates + ((size_t)(c0 + (okt ? tid : 0)) * N + hd) * KTX_MLSTM_GATE_FLOATS;
+      rg[0] = okt ? g[3] : 0.f;
+      rg[1] = okt ? g[4] : 0.f;
+      rg[2] = okt ? g[5] : 0.f;
+      rg[3] = okt ? g[2] : 1.f;
+      rg[4] = okt ? g[6] : 0.f;
+      rg[5] = nv > 0 ? g[7] : 1.f;          // (token 0 of the chunk carries the chunk's decay like every other)
     }
   };
   fetch(t0);
@@ -593,30 +612,14 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, co
 #pragma unroll
     for (int i = 0; i < 4; i++) Vs[tid + i * 256] = rv[i];
     if (tid < ML_CL) {
-      gl[tid] = rg[0];
-      gl[16 + tid] = rg[1];
-      gl[32 + tid] = rg[2];
+      gl[48 + tid] = rg[0];                  // row term
+      gl[64 + tid] = rg[1];                  // column term
+      gl[80 + tid] = rg[2];                  // carry of the incoming state into token t
+      gl[96 + tid] = rg[3];                  // exp(-m_t)
+      gl[112 + tid] = rg[4];                 // weight of token s in the outgoing state
+      if (tid == 0) gl[128] = rg[5];
     }
     if (c0 + ML_CL < t1) fetch(c0 + ML_CL);
-    __syncthreads();
-    if (tid < ML_CL) {
-      float F = 0.f, FL = 0.f;
-      for (int r = 0; r < nv; r++) {
-        FL += gl[r];
-        if (r <= tid) F = FL;
-      }
-      const float mt = gl[32 + tid], zi = gl[16 + tid], mL = gl[32 + nv - 1];
-      const bool ok = tid < nv;
-      gl[48 + tid] = F - mt;                                   // row term of the weights
-      gl[64 + tid] = F - zi;                                   // column term
-      gl[80 + tid] = ok ? expf(F + m0 - mt) : 0.f;             // carry of the incoming state into token t
-      gl[96 + tid] = expf(-mt);
-      gl[112 + tid] = ok ? expf(FL - F + zi - mL) : 0.f;       // weight of token s in the outgoing state
-      if (tid == 0) {
-        gl[128] = expf(FL + m0 - mL);
-        gl[129] = mL;
-      }
-    }
     __syncthreads();
     const float decay = gl[128];
     // (i) A = Q K^T, (ii) weights, row sums, relayout through the wavefront's LDS tile
@@ -702,7 +705,6 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(ktx_mlstm_config c, co
       for (int s2 = 0; s2 < nv; s2++) a += gl[112 + s2] * Ks[s2 * QST + d];
       n_nxt[d] = a;
     }
-    m0 = gl[129];
   }
   __syncthreads();
   for (int e = tid; e < Dp * 64; e += 256) {
