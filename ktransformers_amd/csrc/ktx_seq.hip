@@ -1,6 +1,8 @@
 // ktx_seq.hip — sequence-mixer kernels behind include/ktx_seq.h: sinusoidal embedding, a shape-agnostic dense GEMM (bf16 or
-// fp32 MFMA), sigmoid-weighted grouped-query attention with head mixing over a paged key cache (values = un-normed keys), the
-// mLSTM matrix-memory recurrence over state slots, and the fp32 RMS-norm glue that adds into the residual stream.
+// fp32 MFMA) with its decode-sized streaming forms, sigmoid-weighted grouped-query attention with head mixing over a paged key cache
+// (values = un-normed keys; a matrix-core kernel for prompts and decode steps, a vector-ALU kernel for every other shape and for fp32),
+// the mLSTM matrix-memory recurrence over state slots (gate scan, token-by-token kernel, 16-token chunk kernel on the fp32 matrix
+// cores), and the fp32 RMS-norm glue that adds into the residual stream.
 //
 // Everything a recurrence or a score touches is fp32: the residual, norms, scores, attention weights and their mixing, gates,
 // exponentials and the state.  Element types only select how weights, activations and the key cache are stored and which MFMA

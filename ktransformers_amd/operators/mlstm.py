@@ -51,7 +51,9 @@ class KMLSTMMixer(BaseInjectedModule):
         if self._cfg is None:
             object.__setattr__(self, "_cfg", mlstm_config(self.heads, self.dim, self.vdim, self.gate_cap, self.eps, self.denom_eps))
         if proj is None:
-            proj, base = dense_gemm(h, torch.cat([self.w[n] for n in self.IN_ORDER])), 0
+            if "in" not in self.w:       # used on its own: all input projections as one product
+                self.w["in"] = torch.cat([self.w[n] for n in self.IN_ORDER]).contiguous()
+            proj, base = dense_gemm(h, self.w["in"]), 0
         offs, c = {}, base
         for n, rows in self.in_weight_names():
             offs[n] = c

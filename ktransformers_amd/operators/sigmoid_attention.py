@@ -61,7 +61,9 @@ class KSigmoidTalkAttention(BaseInjectedModule):
         Returns W_o(attention) as fp32 [T, width]."""
         from ktransformers_amd._native_seq import dense_gemm, sigattn_forward, sigattn_prefill, sigattn_prefill_eligible, sigattn_prep
         if proj is None:
-            proj = dense_gemm(h, torch.cat([self.w["q"], self.w["k"]]) if "qk" not in self.w else self.w["qk"])
+            if "qk" not in self.w:       # used on its own: the two input projections as one product
+                self.w["qk"] = torch.cat([self.w["q"], self.w["k"]]).contiguous()
+            proj = dense_gemm(h, self.w["qk"])
             q_off, k_off = 0, self.heads * self.dim
         cfg = self._config(cache)
         kc, kinv = cache.k_caches[self.layer_idx], cache.k_inv[self.layer_idx]
