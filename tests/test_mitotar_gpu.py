@@ -119,9 +119,10 @@ def _attn_case(seed, H, G, D, T, width=32, coef=0.5, every=4, scale=None, pb_mea
     return c, P, h
 
 
-def _run_attention(c, P, h, dtype, chunks, page_size=8, nsplit=None, eps=1e-5):
-    """The operator's kernels on one request whose tokens arrive in `chunks`; returns the attention output before W_o."""
-    from ktransformers_amd._native_seq import dense_gemm, sigattn_config, sigattn_forward, sigattn_prep
+def _run_attention(c, P, h, dtype, chunks, page_size=8, nsplit=None, eps=1e-5, matrix_core=False):
+    """The operator's kernels on one request whose tokens arrive in `chunks`; returns the attention output before W_o.
+    matrix_core: the MFMA kernel (bf16) instead of the vector-ALU one."""
+    from ktransformers_amd._native_seq import dense_gemm, sigattn_config, sigattn_forward, sigattn_prefill, sigattn_prep
     from ktransformers_amd.models.custom_cache import KHybridCache
     H, G, D = c["heads"], c["kv_heads"], c["dim"]
     cache = KHybridCache([{"attn": (G, D), "rec": None}], 4096, max_requests=2, page_size=page_size, dtype=dtype, device=DEV)
@@ -134,8 +135,12 @@ def _run_attention(c, P, h, dtype, chunks, page_size=8, nsplit=None, eps=1e-5):
         fb = cache.plan([("r", n)])
         proj = dense_gemm(h[at:at + n].float().to(DEV), w_in)
         q = sigattn_prep(cfg, proj, 0, H * D, f("a.q.norm"), f("a.k.norm"), eps, fb.positions, fb.cache_loc, cache.k_caches[0], cache.k_inv[0])
-        outs.append(sigattn_forward(cfg, q, cache.k_caches[0], cache.k_inv[0], fb.tok_req, fb.positions, fb.page_indptr, fb.page_indices,
-                                    f("a.pb"), f("a.talk"), nsplit=nsplit or fb.nsplit))
+        if matrix_core:
+            outs.append(sigattn_prefill(cfg, q, cache.k_caches[0], cache.k_inv[0], fb.q_indptr, fb.pos0, fb.page_indptr, fb.page_indices,
+                                        f("a.pb"), f("a.talk"), fb.max_q_len, nsplit=nsplit or (1 if n > 1 else 7)).float())
+        else:
+            outs.append(sigattn_forward(cfg, q, cache.k_caches[0], cache.k_inv[0], fb.tok_req, fb.positions, fb.page_indptr, fb.page_indices,
+                                        f("a.pb"), f("a.talk"), nsplit=nsplit or fb.nsplit))
         at += n
     return torch.cat(outs)
 
@@ -223,6 +228,9 @@ def test_one_key_stands_out(dtype, key_at):
     for chunks in ([T], [T - 1, 1]):
         got = _run_attention(c, P, h, dtype, chunks, page_size=8)
         assert rel(got[-1], ref[-1]) < TOL[dtype], (key_at, chunks)
+        if dtype == BF16:       # and through the matrix-core kernel: 32-key tiles, key ranges shared by workgroups in the decode step
+            got = _run_attention(c, P, h, dtype, chunks, page_size=8, matrix_core=True)
+            assert rel(got[-1], ref[-1]) < TOL[dtype], (key_at, chunks, "matrix cores")
     alone = _ref_attention(c, P, h[T - 1:])          # the query's pair with itself only
     assert (ref[-1] - alone[0]).abs().max() > 1.0      # the far key does carry weight in the plain statement
 
