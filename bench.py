@@ -1601,9 +1601,9 @@ def run_mitotar(args, dev):
         sz = MITOTAR_SIZES[name]
         layer = {"type": "parallel", "mlp": {"kind": "dense", "ff": sz["ff"]},
                  "mixer": {"left": {"heads": sz["heads"], "kv_heads": sz["kv_heads"], "dim": sz["dim"], "vdim": sz["dim"],
-                                    "scale": sz["dim"] ** -0.5, "q_temp": {"coef": 0.5, "every": 64}},
-                           "right": {"heads": sz["r_heads"], "dim": sz["r_dim"], "vdim": sz["r_vdim"], "gate_cap": 12.0}}}
-        cfg = {"architecture": "Mitotar", "width": sz["width"], "vocab": 32000, "norm": {"eps": 1e-6}, "layers": [layer] * n_layers}
+                                    "scale": sz["dim"] ** -0.5, "q_temp": {"coef": 0.4, "every": 128}},
+                           "right": {"heads": sz["r_heads"], "dim": sz["r_dim"], "vdim": sz["r_vdim"], "gate_cap": 15.0}}}
+        cfg = {"architecture": "Mitotar", "width": sz["width"], "vocab": 32000, "norm": {"eps": 1e-5}, "layers": [layer] * n_layers}
         with contextlib.redirect_stdout(io.StringIO()):
             model, config, entry = load_model(cfg, dtype=torch.bfloat16, device=str(dev), loader=SeqRandomLoader(cfg, dev))
         cache = entry.make_cache(config, 8 * (ctx + 64) + T, 16, torch.bfloat16, str(dev))
