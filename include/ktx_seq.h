@@ -27,7 +27,8 @@ enum { KTX_SEQ_F32 = 0, KTX_SEQ_BF16 = 1 };
 enum { KTX_ACT_NONE = 0, KTX_ACT_GELU_TANH = 1 };
 
 /* x[t] = embed[tokens[t]] + s(pos[t]),  s(p)[2i] = sin(p * inv_freq[i]),  s(p)[2i+1] = cos(p * inv_freq[i]).
- * inv_freq: fp64 [(width + 1) / 2]; the angle and its sine are evaluated in fp64 and rounded once.  x: fp32 [T][width]. */
+ * inv_freq: fp64 [(width + 1) / 2]; the angle and its sine are evaluated in fp64 and rounded once.  x: fp32 [T][width].
+ * d_inv_freq == NULL: x[t] = embed[tokens[t]] alone (d_pos is not read). */
 int ktx_embed_sinpos(int T, int width, int vocab, const int32_t* d_tokens, const int32_t* d_pos, const void* d_embed,
                      int embed_dtype, const double* d_inv_freq, float* d_x, ktx_stream_t stream);
 

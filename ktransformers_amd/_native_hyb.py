@@ -1,0 +1,269 @@
+"""ctypes binding of include/ktx_hyb.h — the hybrid-decoder kernels (layer norm with bias, the gated post-normed residual update,
+PolyNorm, the gated delta rule over state slots, sliding-window softmax attention with a sink over a paged latent cache, the sigmoid
+top-k router, the expert sort and the grouped GEMM).  Same library and calling rules as ktransformers_amd._native_seq: device
+pointers and the caller's current HIP stream cross the boundary, every call is graph-capturable, there is no CPU fallback."""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from ktransformers_amd._native_seq import SEQ_DTYPE, KtxError, _seq_dev, _stream_ptr, check, lib
+
+
+class _DeltaConfig(C.Structure):     # include/ktx_hyb.h: ktx_delta_config
+    _fields_ = [("heads", C.c_int32), ("kv_heads", C.c_int32), ("dim", C.c_int32), ("vdim", C.c_int32), ("taps", C.c_int32),
+                ("unit_eps", C.c_float)]
+
+
+class _LatAttnConfig(C.Structure):   # include/ktx_hyb.h: ktx_latattn_config
+    _fields_ = [("heads", C.c_int32), ("dim", C.c_int32), ("rot_dim", C.c_int32), ("vdim", C.c_int32), ("kv_rank", C.c_int32),
+                ("rot_dims", C.c_int32), ("scale", C.c_float), ("window", C.c_int32), ("eps", C.c_float), ("page_size", C.c_int32),
+                ("cache_dtype", C.c_int32)]
+
+
+_P, _I, _L, _F = C.c_void_p, C.c_int, C.c_int64, C.c_float
+if not hasattr(lib, "ktx_grouped_gemm"):
+    raise ImportError("the loaded kernel library predates include/ktx_hyb.h: rebuild with `python -m ktransformers_amd.build [--seq]`")
+lib.ktx_rows_add.argtypes = [_I, _I, _P, _P, _P, _P]
+lib.ktx_layer_norm.argtypes = [_I, _I, _P, _P, _P, _F, _P, _P, _I, _P]
+lib.ktx_gated_norm_add.argtypes = [_I, _I, _P, _L, _P, _P, _P, _P, _I, _P, _L, _P, _P, _P, _F, _P, _P]
+lib.ktx_poly_norm.argtypes = [_I, _I, _P, _L, _P, _P, _F, _P, _I, _P]
+lib.ktx_silu_mul_rows.argtypes = [_I, _I, _P, _L, _P, _I, _P]
+lib.ktx_head_gate_norm.argtypes = [_I, _I, _I, _F, _P, _P, _L, _P, _I, _I, _P, _I, _P]
+lib.ktx_delta_prep.argtypes = [C.POINTER(_DeltaConfig), _I, _I, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P]
+lib.ktx_delta_forward.argtypes = [C.POINTER(_DeltaConfig), _I, _P, _P, _P, _P, _P, _P, _P, _P]
+lib.ktx_latattn_prep.argtypes = [C.POINTER(_LatAttnConfig), _I, _P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P]
+lib.ktx_latattn_forward.argtypes = [C.POINTER(_LatAttnConfig), _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _P]
+lib.ktx_moe_route.argtypes = [_I, _I, _I, _F, _F, _P, _L, _P, _P, _P]
+lib.ktx_moe_plan.argtypes = [_I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P]
+lib.ktx_grouped_gemm.argtypes = [_I, _I, _I, _I, _P, _I, _L, _L, _P, _P, _I, _P, _I, _L, _L, _P, _P, _P, _P, _I, _P]
+
+TILE_M = 64
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None else None
+
+
+def _f32(t, what):
+    return None if t is None else _seq_dev(t, torch.float32, what)
+
+
+def _i32(t, what):
+    return None if t is None else _seq_dev(t, torch.int32, what)
+
+
+def _rows_f32(t, what):
+    """fp32 rows with unit inner stride (a column slice of a GEMM's output is fine) -> (pointer, row stride)."""
+    if t is None:
+        return None, 0
+    if not t.is_cuda or t.dtype != torch.float32 or t.dim() != 2 or t.stride(1) != 1:
+        raise KtxError(f"{what}: expected fp32 rows on a HIP device, got {t.dtype} {tuple(t.shape)} strides {t.stride()}")
+    return t.data_ptr(), t.stride(0)
+
+
+def rows_add(x: torch.Tensor, x0: torch.Tensor | None = None, vec: torch.Tensor | None = None) -> torch.Tensor:
+    """x[t] += x0[t] + vec, in place (ktx_rows_add)."""
+    _f32(x, "rows_add x"), _f32(x0, "rows_add x0"), _f32(vec, "rows_add vec")
+    T, W = x.shape
+    if (x0 is not None and x0.shape != x.shape) or (vec is not None and vec.numel() != W):
+        raise KtxError("rows_add: shapes do not fit")
+    check(lib.ktx_rows_add(T, W, x.data_ptr(), _ptr(x0), _ptr(vec), _stream_ptr(x.device)))
+    return x
+
+
+def layer_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None, eps: float, rows: torch.Tensor | None = None,
+               out_dtype=torch.float32) -> torch.Tensor:
+    _f32(x, "layer_norm x"), _f32(w, "layer_norm w"), _f32(b, "layer_norm b"), _i32(rows, "layer_norm rows")
+    W = x.shape[-1]
+    T = rows.numel() if rows is not None else x.numel() // W
+    if w.numel() != W or (b is not None and b.numel() != W):
+        raise KtxError("layer_norm: weight / bias do not fit the row")
+    out = torch.empty((T, W), dtype=out_dtype, device=x.device)
+    check(lib.ktx_layer_norm(T, W, x.data_ptr(), w.data_ptr(), _ptr(b), float(eps), _ptr(rows), out.data_ptr(), SEQ_DTYPE[out_dtype],
+                             _stream_ptr(x.device)))
+    return out
+
+
+def gated_norm_add(x: torch.Tensor, wn: torch.Tensor, bn: torch.Tensor | None, eps: float, y: torch.Tensor | None = None,
+                   ybias: torch.Tensor | None = None, gate_logits: torch.Tensor | None = None, gate_bias: torch.Tensor | None = None,
+                   expert_rows: torch.Tensor | None = None, pair_pos: torch.Tensor | None = None, topk_w: torch.Tensor | None = None
+                   ) -> torch.Tensor:
+    """x += layer_norm((y + ybias + sum_k topk_w[t, k] expert_rows[pair_pos[t, k]]) * sigmoid(gate_logits + gate_bias)), in place."""
+    _f32(x, "gated_norm_add x"), _f32(wn, "wn"), _f32(bn, "bn"), _f32(ybias, "ybias"), _f32(gate_bias, "gate_bias")
+    _f32(expert_rows, "expert_rows"), _i32(pair_pos, "pair_pos"), _f32(topk_w, "topk_w")
+    T, W = x.shape
+    yp, ldy = _rows_f32(y, "gated_norm_add y")
+    gp, ldg = _rows_f32(gate_logits, "gated_norm_add gate_logits")
+    for t in (y, gate_logits):
+        if t is not None and tuple(t.shape) != (T, W):
+            raise KtxError("gated_norm_add: y / gate_logits must be [T, W]")
+    top = 0
+    if expert_rows is not None:
+        top = topk_w.shape[1]
+        if expert_rows.shape[1] != W or pair_pos.numel() != T * top or topk_w.shape[0] != T:
+            raise KtxError("gated_norm_add: the gathered term does not fit")
+    check(lib.ktx_gated_norm_add(T, W, yp, ldy, _ptr(ybias), _ptr(expert_rows), _ptr(pair_pos), _ptr(topk_w), top, gp, ldg, _ptr(gate_bias),
+                                 wn.data_ptr(), _ptr(bn), float(eps), x.data_ptr(), _stream_ptr(x.device)))
+    return x
+
+
+def poly_norm(z: torch.Tensor, bias: torch.Tensor | None, coef: torch.Tensor, eps: float, out_dtype=torch.float32) -> torch.Tensor:
+    zp, ldz = _rows_f32(z, "poly_norm z")
+    _f32(bias, "poly_norm bias"), _f32(coef, "poly_norm coef")
+    T, F = z.shape
+    if coef.numel() != 4 or (bias is not None and bias.numel() != F):
+        raise KtxError("poly_norm: four coefficients, a bias per entry")
+    out = torch.empty((T, F), dtype=out_dtype, device=z.device)
+    check(lib.ktx_poly_norm(T, F, zp, ldz, _ptr(bias), coef.data_ptr(), float(eps), out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(z.device)))
+    return out
+
+
+def silu_mul_rows(gu: torch.Tensor, out_dtype=torch.float32) -> torch.Tensor:
+    """[R, 2F] (gate | up) -> silu(gate) * up, [R, F]."""
+    p, ld = _rows_f32(gu, "silu_mul_rows")
+    R, F = gu.shape[0], gu.shape[1] // 2
+    out = torch.empty((R, F), dtype=out_dtype, device=gu.device)
+    check(lib.ktx_silu_mul_rows(R, F, p, ld, out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(gu.device)))
+    return out
+
+
+def head_gate_norm(o: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, heads: int, vdim: int, eps: float, w_per_head: bool, act: str,
+                   out_dtype=torch.float32) -> torch.Tensor:
+    _f32(o, "head_gate_norm o"), _f32(w, "head_gate_norm w")
+    gp, ldg = _rows_f32(gate, "head_gate_norm gate")
+    T = o.shape[0]
+    if o.numel() != T * heads * vdim or gate.shape[1] != heads * vdim or w.numel() != (heads * vdim if w_per_head else vdim):
+        raise KtxError("head_gate_norm: shapes do not fit")
+    out = torch.empty((T, heads * vdim), dtype=out_dtype, device=o.device)
+    check(lib.ktx_head_gate_norm(T, heads, vdim, float(eps), o.data_ptr(), gp, ldg, w.data_ptr(), int(w_per_head),
+                                 {"sigmoid": 0, "silu": 1}[act], out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(o.device)))
+    return out
+
+
+def delta_config(heads: int, kv_heads: int, dim: int, vdim: int, taps: int, unit_eps: float) -> _DeltaConfig:
+    return _DeltaConfig(heads, kv_heads, dim, vdim, int(taps), float(unit_eps))
+
+
+def delta_prep(cfg: _DeltaConfig, proj: torch.Tensor, offs: dict, taps: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor,
+               batch, conv_state: torch.Tensor | None):
+    """-> (qkv fp32 [T, C], gb fp32 [T, 2 heads]); the slots' convolution state moves on (ktx_delta_prep)."""
+    pp, ldp = _rows_f32(proj, "delta_prep proj")
+    _f32(taps, "taps"), _f32(A_log, "A_log"), _f32(dt_bias, "dt_bias"), _f32(conv_state, "conv_state")
+    T = proj.shape[0]
+    Cn = 2 * cfg.kv_heads * cfg.dim + cfg.heads * cfg.vdim
+    if tuple(taps.shape) != (Cn, cfg.taps) or A_log.numel() != cfg.heads or dt_bias.numel() != cfg.heads:
+        raise KtxError("delta_prep: taps [C, taps], A_log / dt_bias [heads]")
+    if conv_state is not None and tuple(conv_state.shape[1:]) != (max(cfg.taps - 1, 1), Cn):
+        raise KtxError("delta_prep: conv_state must be [slots, taps - 1, C]")
+    qkv = torch.empty((T, Cn), dtype=torch.float32, device=proj.device)
+    gb = torch.empty((T, 2 * cfg.heads), dtype=torch.float32, device=proj.device)
+    check(lib.ktx_delta_prep(C.byref(cfg), batch.B, T, batch.q_indptr.data_ptr(), batch.pos0.data_ptr(), batch.slot.data_ptr(),
+                             batch.tok_req.data_ptr(), pp, ldp, offs["q"], offs["k"], offs["v"], offs["b"], offs["a"], taps.data_ptr(),
+                             A_log.data_ptr(), dt_bias.data_ptr(), _ptr(conv_state), qkv.data_ptr(), gb.data_ptr(), _stream_ptr(proj.device)))
+    return qkv, gb
+
+
+def delta_forward(cfg: _DeltaConfig, qkv: torch.Tensor, gb: torch.Tensor, batch, S: torch.Tensor) -> torch.Tensor:
+    _f32(qkv, "delta_forward qkv"), _f32(gb, "delta_forward gb"), _f32(S, "delta_forward S")
+    if tuple(S.shape[1:]) != (cfg.heads, cfg.dim, cfg.vdim):
+        raise KtxError("delta_forward: S must be [slots, heads, dim, vdim]")
+    T = qkv.shape[0]
+    o = torch.empty((T, cfg.heads * cfg.vdim), dtype=torch.float32, device=qkv.device)
+    check(lib.ktx_delta_forward(C.byref(cfg), batch.B, batch.q_indptr.data_ptr(), batch.pos0.data_ptr(), batch.slot.data_ptr(),
+                                qkv.data_ptr(), gb.data_ptr(), S.data_ptr(), o.data_ptr(), _stream_ptr(qkv.device)))
+    return o
+
+
+def latattn_config(heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, rot_dims: int, scale: float, window: int, eps: float,
+                   page_size: int, cache_dtype) -> _LatAttnConfig:
+    return _LatAttnConfig(heads, dim, rot_dim, vdim, kv_rank, int(rot_dims), float(scale), int(window), float(eps), int(page_size),
+                          SEQ_DTYPE[cache_dtype])
+
+
+def latattn_prep(cfg: _LatAttnConfig, proj: torch.Tensor, q_off: int, c_off: int, wn: torch.Tensor, inv_freq: torch.Tensor,
+                 positions: torch.Tensor, cache_loc: torch.Tensor, cache: torch.Tensor, q_out: torch.Tensor) -> None:
+    pp, ldp = _rows_f32(proj, "latattn_prep proj")
+    _f32(wn, "latattn_prep wn"), _f32(q_out, "latattn_prep q_out"), _i32(positions, "positions"), _i32(cache_loc, "cache_loc")
+    _seq_dev(inv_freq, torch.float64, "latattn_prep inv_freq")
+    T, E = proj.shape[0], cfg.kv_rank + cfg.rot_dim
+    if positions.numel() != T or cache_loc.numel() != T or cache.shape[-1] != E or q_out.numel() != T * cfg.heads * E or \
+            inv_freq.numel() != cfg.rot_dims // 2 or wn.numel() != cfg.kv_rank or not cache.is_contiguous():
+        raise KtxError("latattn_prep: shapes do not fit")
+    check(lib.ktx_latattn_prep(C.byref(cfg), T, pp, ldp, q_off, c_off, wn.data_ptr(), inv_freq.data_ptr(), positions.data_ptr(),
+                               cache_loc.data_ptr(), cache.data_ptr(), q_out.data_ptr(), _stream_ptr(proj.device)))
+
+
+def latattn_forward(cfg: _LatAttnConfig, q: torch.Tensor, cache: torch.Tensor, batch, sink: torch.Tensor, nsplit: int = 1,
+                    out_dtype=torch.float32) -> torch.Tensor:
+    """-> [T, heads * kv_rank] of out_dtype: each head's softmax-weighted sum of latent rows (ktx_latattn_forward)."""
+    _f32(q, "latattn_forward q"), _f32(sink, "latattn_forward sink")
+    T, L = q.shape[0], cfg.kv_rank
+    out = torch.empty((T, cfg.heads * L), dtype=out_dtype, device=q.device)
+    scratch = torch.empty((nsplit, T, cfg.heads, L + 2), dtype=torch.float32, device=q.device) if nsplit > 1 else None
+    check(lib.ktx_latattn_forward(C.byref(cfg), T, q.data_ptr(), cache.data_ptr(), batch.tok_req.data_ptr(), batch.positions.data_ptr(),
+                                  batch.page_indptr.data_ptr(), batch.page_indices.data_ptr(), sink.data_ptr(), int(nsplit), _ptr(scratch),
+                                  out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(q.device)))
+    return out
+
+
+def moe_route(logits: torch.Tensor, top: int, scale: float, sum_eps: float):
+    """logits fp32 rows [T, E] -> (topk_idx int32 [T, top], topk_w fp32 [T, top]) (ktx_moe_route)."""
+    lp, ldl = _rows_f32(logits, "moe_route logits")
+    T, E = logits.shape
+    idx = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    check(lib.ktx_moe_route(T, E, top, float(scale), float(sum_eps), lp, ldl, idx.data_ptr(), w.data_ptr(), _stream_ptr(logits.device)))
+    return idx, w
+
+
+class MoePlan:
+    __slots__ = ("group_off", "sorted_tok", "pair_pos", "tile_group", "tile_row0", "num_tiles", "max_tiles", "pairs")
+
+
+def moe_plan(topk_idx: torch.Tensor, E: int) -> MoePlan:
+    _i32(topk_idx, "moe_plan topk_idx")
+    T, top = topk_idx.shape
+    p = MoePlan()
+    p.pairs = T * top
+    p.max_tiles = p.pairs // TILE_M + min(E, p.pairs) + 1
+    meta = torch.empty(E + 1 + 2 * p.pairs + 2 * p.max_tiles + 1, dtype=torch.int32, device=topk_idx.device)
+    at = 0
+    for name, n in (("group_off", E + 1), ("sorted_tok", p.pairs), ("pair_pos", p.pairs), ("tile_group", p.max_tiles),
+                    ("tile_row0", p.max_tiles), ("num_tiles", 1)):
+        setattr(p, name, meta[at:at + n])
+        at += n
+    check(lib.ktx_moe_plan(T, E, top, TILE_M, topk_idx.data_ptr(), p.group_off.data_ptr(), p.sorted_tok.data_ptr(), p.pair_pos.data_ptr(),
+                           p.tile_group.data_ptr(), p.tile_row0.data_ptr(), p.num_tiles.data_ptr(), _stream_ptr(topk_idx.device)))
+    return p
+
+
+def _gg_types(a, w, out_dtype):
+    if a.dtype not in SEQ_DTYPE or w.dtype not in SEQ_DTYPE or not a.is_cuda or a.stride(-1) != 1 or not w.is_contiguous():
+        raise KtxError(f"grouped_gemm: {a.dtype} {tuple(a.shape)} x {w.dtype} {tuple(w.shape)} does not fit")
+    if w.dtype == torch.float32 and (a.dtype != torch.float32 or out_dtype != torch.float32):
+        raise KtxError("grouped_gemm: an fp32 product takes and writes fp32")
+
+
+def head_gemm(a: torch.Tensor, a_goff: int, w: torch.Tensor, out: torch.Tensor, y_goff: int) -> torch.Tensor:
+    """Per-head products: for g < G, out[:, g * y_goff : g * y_goff + N] = a[:, g * a_goff : g * a_goff + K] @ w[g]^T
+    (w [G, N, K]; a, out 2-D rows whose columns may start anywhere — pass the views)."""
+    G, N, K = w.shape
+    _gg_types(a, w, out.dtype)
+    M = a.shape[0]
+    check(lib.ktx_grouped_gemm(G, M, N, K, a.data_ptr(), SEQ_DTYPE[a.dtype], a.stride(0), a_goff, None, w.data_ptr(), SEQ_DTYPE[w.dtype],
+                               out.data_ptr(), SEQ_DTYPE[out.dtype], out.stride(0), y_goff, None, None, None, None, 0, _stream_ptr(a.device)))
+    return out
+
+
+def expert_gemm(a: torch.Tensor, w: torch.Tensor, plan: MoePlan, gather: bool, out_dtype=torch.float32) -> torch.Tensor:
+    """Sorted row r (expert g = the group it falls in) : out[r] = a[plan.sorted_tok[r] if gather else r] @ w[g]^T.  w [E, N, K]."""
+    G, N, K = w.shape
+    _gg_types(a, w, out_dtype)
+    out = torch.empty((plan.pairs, N), dtype=out_dtype, device=a.device)
+    check(lib.ktx_grouped_gemm(G, plan.pairs, N, K, a.data_ptr(), SEQ_DTYPE[a.dtype], a.stride(0), 0,
+                               plan.sorted_tok.data_ptr() if gather else None, w.data_ptr(), SEQ_DTYPE[w.dtype], out.data_ptr(),
+                               SEQ_DTYPE[out_dtype], out.stride(0), 0, plan.group_off.data_ptr(), plan.tile_group.data_ptr(),
+                               plan.tile_row0.data_ptr(), plan.num_tiles.data_ptr(), plan.max_tiles, _stream_ptr(a.device)))
+    return out

@@ -93,6 +93,18 @@ def embed_sinpos(tokens: torch.Tensor, positions: torch.Tensor, embed: torch.Ten
     return x
 
 
+def embed_rows(tokens: torch.Tensor, embed: torch.Tensor) -> torch.Tensor:
+    """tokens int32 [T]; embed [vocab, width] bf16 | fp32 -> the table rows as fp32 [T, width] (ktx_embed_sinpos without positions)."""
+    _seq_dev(tokens, torch.int32, "embed_rows tokens"), _seq_dev(embed, None, "embed_rows embed")
+    if embed.dtype not in SEQ_DTYPE:
+        raise KtxError("embed_rows: element type does not fit")
+    T, (vocab, width) = tokens.numel(), embed.shape
+    x = torch.empty((T, width), dtype=torch.float32, device=tokens.device)
+    check(lib.ktx_embed_sinpos(T, width, vocab, tokens.data_ptr(), None, embed.data_ptr(), SEQ_DTYPE[embed.dtype], None, x.data_ptr(),
+                               _stream_ptr(x.device)))
+    return x
+
+
 def dense_gemm(a: torch.Tensor, w: torch.Tensor, out_dtype=torch.float32, act: str | None = None, out: torch.Tensor | None = None,
                ksplit: int = 1) -> torch.Tensor:
     """a [M, K] (fp32 | bf16, unit inner stride) x w [N, K]^T (contiguous bf16 | fp32: its type is the product's) -> [M, N] of

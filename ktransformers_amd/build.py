@@ -18,9 +18,10 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(LIBDIR, "obj")
 LIB = os.path.join(LIBDIR, "libktx_hip.so")
-# the sequence-mixer kernels alone (include/ktx_seq.h): what a model without MoE / MLA layers needs, built in seconds
+# the sequence-mixer and hybrid-decoder kernels alone (include/ktx_seq.h, ktx_hyb.h): what the fp32-residual families need, built in
+# well under a minute
 SEQ_LIB = os.path.join(LIBDIR, "libktx_seq.so")
-SEQ_SOURCES = ("ktx_seq.hip", "ktx_err.hip")
+SEQ_SOURCES = ("ktx_seq.hip", "ktx_hyb.hip", "ktx_err.hip")
 
 # -ffp-contract=off: the parity contract needs every fp32 op rounded exactly as the reference's AVX512 code does;
 # FMAs appear only where the reference issues one (explicit fmaf()).
@@ -29,7 +30,8 @@ CFLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-f
 
 # per-source extra flags: the sequence-mixer kernels keep fp32 state and norms on the vector ALUs and are built without the packed
 # fp32 instructions (scalar v_fma / v_mul only)
-EXTRA_CFLAGS = {"ktx_seq.hip": ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]}
+_NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+EXTRA_CFLAGS = {"ktx_seq.hip": _NO_PACKED_FP32, "ktx_hyb.hip": _NO_PACKED_FP32}
 
 
 def sources() -> list[str]:

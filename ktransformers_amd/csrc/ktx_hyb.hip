@@ -1,0 +1,912 @@
+// ktx_hyb.hip — hybrid-decoder kernels behind include/ktx_hyb.h: layer norm with bias, the sigmoid-gated post-normed residual update
+// (with the mixture's weighted gather folded in), PolyNorm, the gated delta rule (convolution + unit vectors + decay prep, state update,
+// token-by-token recurrence on register-resident state slices), sliding-window softmax attention with a sink over a paged latent cache,
+// the sigmoid top-k router with its expert sort, and a grouped GEMM (per-head products and per-expert products) on the matrix cores.
+//
+// Everything a recurrence, a norm, a router or a score touches is fp32; element types only select how weights, activations and the
+// latent cache are stored and which MFMA multiplies them.
+#include "ktx_common.h"
+#include "../../include/ktx_hyb.h"
+
+#include <math.h>
+
+#include <algorithm>
+
+namespace {
+
+#include "ktx_seq_dev.inc"
+
+__device__ __forceinline__ float silu_f32(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplus_f32(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+// ---------------------------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) rows_add_kernel(size_t n, int W, float* __restrict__ x, const float* __restrict__ x0,
+                                                       const float* __restrict__ vec) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float v = x[i];
+  if (x0) v += x0[i];
+  if (vec) v += vec[i % W];
+  x[i] = v;
+}
+
+// layer norm of one row per workgroup: mean, then the mean of squared deviations, then the affine map
+template <typename OT>
+__global__ void __launch_bounds__(256) layer_norm_kernel(int W, const float* __restrict__ x, const float* __restrict__ w,
+                                                         const float* __restrict__ b, float eps, const int32_t* __restrict__ rows,
+                                                         OT* __restrict__ out) {
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const float* a = x + (size_t)(rows ? rows[t] : t) * W;
+  float s = 0.f;
+  for (int e = tid; e < W; e += 256) s += a[e];
+  const float mean = block_sum256(s, red) / (float)W;
+  float q = 0.f;
+  for (int e = tid; e < W; e += 256) {
+    const float d = a[e] - mean;
+    q += d * d;
+  }
+  const float r = 1.0f / sqrtf(block_sum256(q, red) / (float)W + eps);
+  for (int e = tid; e < W; e += 256) st_elem(out, (size_t)t * W + e, (a[e] - mean) * r * w[e] + (b ? b[e] : 0.f));
+}
+
+// z = (y + ybias + sum_k w_k ey[pos_k]) * sigmoid(gl + gbias); x += LN(z).  The row lives in LDS between the passes.
+__global__ void __launch_bounds__(256) gated_norm_add_kernel(int W, const float* __restrict__ y, int64_t ldy,
+                                                             const float* __restrict__ ybias, const float* __restrict__ ey,
+                                                             const int32_t* __restrict__ pair_pos, const float* __restrict__ topk_w,
+                                                             int top, const float* __restrict__ gl, int64_t ldg,
+                                                             const float* __restrict__ gbias, const float* __restrict__ wn,
+                                                             const float* __restrict__ bn, float eps, float* __restrict__ x) {
+  extern __shared__ float zrow[];
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  float s = 0.f;
+  for (int e = tid; e < W; e += 256) {
+    float z = y ? y[(size_t)t * ldy + e] : 0.f;
+    if (ybias) z += ybias[e];
+    if (ey) {
+      float m = 0.f;
+      for (int k = 0; k < top; k++) m += topk_w[(size_t)t * top + k] * ey[(size_t)pair_pos[(size_t)t * top + k] * W + e];
+      z += m;
+    }
+    if (gl) z *= sigmoid_f32(gl[(size_t)t * ldg + e] + (gbias ? gbias[e] : 0.f));
+    zrow[e] = z;
+    s += z;
+  }
+  const float mean = block_sum256(s, red) / (float)W;
+  float q = 0.f;
+  for (int e = tid; e < W; e += 256) {
+    const float d = zrow[e] - mean;
+    q += d * d;
+  }
+  const float r = 1.0f / sqrtf(block_sum256(q, red) / (float)W + eps);
+  for (int e = tid; e < W; e += 256) x[(size_t)t * W + e] += (zrow[e] - mean) * r * wn[e] + (bn ? bn[e] : 0.f);
+}
+
+template <typename OT>
+__global__ void __launch_bounds__(256) poly_norm_kernel(int F, const float* __restrict__ zin, int64_t ldz, const float* __restrict__ bias,
+                                                        const float* __restrict__ coef, float eps, OT* __restrict__ out) {
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const float* a = zin + (size_t)t * ldz;
+  float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  for (int e = tid; e < F; e += 256) {
+    const float z = a[e] + (bias ? bias[e] : 0.f), z2 = z * z;
+    s1 += z2;
+    s2 += z2 * z2;
+    s3 += z2 * z2 * z2;
+  }
+  const float r1 = coef[0] / sqrtf(block_sum256(s1, red) / (float)F + eps);
+  const float r2 = coef[1] / sqrtf(block_sum256(s2, red) / (float)F + eps);
+  const float r3 = coef[2] / sqrtf(block_sum256(s3, red) / (float)F + eps);
+  const float c3 = coef[3];
+  for (int e = tid; e < F; e += 256) {
+    const float z = a[e] + (bias ? bias[e] : 0.f), z2 = z * z;
+    st_elem(out, (size_t)t * F + e, ((z * r1 + z2 * r2) + z2 * z * r3) + c3);
+  }
+}
+
+template <typename OT>
+__global__ void __launch_bounds__(256) silu_mul_rows_kernel(size_t n, int F, const float* __restrict__ in, int64_t ldi,
+                                                            OT* __restrict__ out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const size_t r = i / F, f = i % F;
+  st_elem(out, i, silu_f32(in[r * ldi + f]) * in[r * ldi + F + f]);
+}
+
+// one workgroup per token; a wavefront takes heads wave, wave + 4, ...
+template <typename OT>
+__global__ void __launch_bounds__(256) head_gate_norm_kernel(int heads, int vdim, float eps, const float* __restrict__ o,
+                                                             const float* __restrict__ gate, int64_t ldg, const float* __restrict__ w,
+                                                             int w_per_head, int act, OT* __restrict__ out) {
+  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int h = wave; h < heads; h += 4) {
+    const float* a = o + ((size_t)t * heads + h) * vdim;
+    float s = 0.f;
+    for (int v = lane; v < vdim; v += 64) s += a[v] * a[v];
+    const float r = 1.0f / sqrtf(wave_sum(s) / (float)vdim + eps);
+    for (int v = lane; v < vdim; v += 64) {
+      const float g = gate[(size_t)t * ldg + h * vdim + v];
+      const float ga = act ? silu_f32(g) : sigmoid_f32(g);
+      st_elem(out, ((size_t)t * heads + h) * vdim + v, a[v] * r * w[(w_per_head ? h * vdim : 0) + v] * ga);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// gated delta rule: prep (one workgroup per token)
+__global__ void __launch_bounds__(256) delta_prep_kernel(ktx_delta_config c, const int32_t* __restrict__ q_indptr,
+                                                         const int32_t* __restrict__ pos0, const int32_t* __restrict__ slot,
+                                                         const int32_t* __restrict__ tok_req, const float* __restrict__ proj, int64_t ldp,
+                                                         int q_off, int k_off, int v_off, int b_off, int a_off,
+                                                         const float* __restrict__ taps, const float* __restrict__ A_log,
+                                                         const float* __restrict__ dt_bias, const float* __restrict__ conv_state,
+                                                         float* __restrict__ qkv, float* __restrict__ gb) {
+  extern __shared__ float ch[];            // [C] convolved, activated channels of this token
+  const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int GD = c.kv_heads * c.dim, C = 2 * GD + c.heads * c.vdim, K = c.taps;
+  const int b = tok_req[t], first = q_indptr[b], i = t - first;
+  const bool carried = pos0[b] > 0;
+  const float* st = conv_state + (size_t)slot[b] * (K - 1) * C;
+  for (int e = tid; e < C; e += 256) {
+    const int col = e < GD ? q_off + e : (e < 2 * GD ? k_off + e - GD : v_off + e - 2 * GD);
+    float acc = 0.f;
+    for (int j = 0; j < K; j++) {          // input i - j times the tap K - 1 - j
+      const int ii = i - j;
+      float v = 0.f;
+      if (ii >= 0) v = proj[(size_t)(first + ii) * ldp + col];
+      else if (carried) v = st[(size_t)(K - 1 + ii) * C + e];
+      acc += taps[(size_t)e * K + (K - 1 - j)] * v;
+    }
+    ch[e] = silu_f32(acc);
+  }
+  __syncthreads();
+  // unit vectors: 2 * kv_heads heads of q | k
+  for (int hh = wave; hh < 2 * c.kv_heads; hh += 4) {
+    float* a = ch + (size_t)hh * c.dim;
+    float s = 0.f;
+    for (int d = lane; d < c.dim; d += 64) s += a[d] * a[d];
+    float r = 1.0f / sqrtf(wave_sum(s) + c.unit_eps);
+    if (hh < c.kv_heads) r *= 1.0f / sqrtf((float)c.dim);
+    for (int d = lane; d < c.dim; d += 64) a[d] *= r;
+  }
+  __syncthreads();
+  for (int e = tid; e < C; e += 256) qkv[(size_t)t * C + e] = ch[e];
+  for (int h = tid; h < c.heads; h += 256) {
+    const float a = proj[(size_t)t * ldp + a_off + h] + dt_bias[h];
+    gb[(size_t)t * 2 * c.heads + h] = expf(-expf(A_log[h]) * softplus_f32(a));
+    gb[(size_t)t * 2 * c.heads + c.heads + h] = sigmoid_f32(proj[(size_t)t * ldp + b_off + h]);
+  }
+}
+
+// the last taps - 1 inputs of every request of the step become its slot's convolution state (thread = request x channel; the old
+// entries it still needs lie ahead of the ones it overwrites)
+__global__ void __launch_bounds__(256) delta_conv_update_kernel(ktx_delta_config c, const int32_t* __restrict__ q_indptr,
+                                                                const int32_t* __restrict__ pos0, const int32_t* __restrict__ slot,
+                                                                const float* __restrict__ proj, int64_t ldp, int q_off, int k_off,
+                                                                int v_off, float* __restrict__ conv_state) {
+  const int GD = c.kv_heads * c.dim, C = 2 * GD + c.heads * c.vdim, K = c.taps;
+  const int b = blockIdx.y, e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= C) return;
+  const int first = q_indptr[b], n = q_indptr[b + 1] - first;
+  if (n <= 0) return;
+  const bool carried = pos0[b] > 0;
+  const int col = e < GD ? q_off + e : (e < 2 * GD ? k_off + e - GD : v_off + e - 2 * GD);
+  float* st = conv_state + (size_t)slot[b] * (K - 1) * C;
+  for (int j = 0; j < K - 1; j++) {
+    const int ii = n - (K - 1) + j;
+    float v = 0.f;
+    if (ii >= 0) v = proj[(size_t)(first + ii) * ldp + col];
+    else if (carried) v = st[(size_t)(j + n) * C + e];
+    st[(size_t)j * C + e] = v;
+  }
+}
+
+// the recurrence: workgroup = (request, head, 64 value columns); wavefront = a quarter of the dim rows, lane = value column; the state
+// slice stays in registers; ONE barrier per token: both read-outs (S^T k and S^T q of the decayed state) are taken before the write,
+// o = (g S)^T q + u (k . q).
+template <int DPW>
+__global__ void __launch_bounds__(256) delta_fwd_kernel(ktx_delta_config c, const int32_t* __restrict__ q_indptr,
+                                                        const int32_t* __restrict__ pos0, const int32_t* __restrict__ slot,
+                                                        const float* __restrict__ qkv, const float* __restrict__ gb,
+                                                        float* __restrict__ Sg, float* __restrict__ o) {
+  constexpr int DP = 4 * DPW;
+  __shared__ float kq[2][2 * DP];          // k | q of the token's key head
+  __shared__ float vv[2][64 + 2];          // the value slice, then g and beta
+  __shared__ float red[2][4][2][64];
+  __shared__ float redkq[2][4];
+  const int VS = (c.vdim + 63) / 64;
+  const int vs = blockIdx.x % VS, h = (blockIdx.x / VS) % c.heads, b = blockIdx.x / (VS * c.heads);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int D = c.dim, V = c.vdim, H = c.heads, GD = c.kv_heads * D, C = 2 * GD + H * V;
+  const int kh = h / (H / c.kv_heads);
+  const int col = vs * 64 + lane;
+  const int t0 = q_indptr[b], t1 = q_indptr[b + 1];
+  if (t1 <= t0) return;
+  float S[DPW];
+  float* Sp = Sg + (((size_t)slot[b] * H + h) * D) * V;
+  const bool carried = pos0[b] > 0;
+#pragma unroll
+  for (int r = 0; r < DPW; r++) {
+    const int d = wave * DPW + r;
+    S[r] = (carried && d < D && col < V) ? Sp[(size_t)d * V + col] : 0.f;
+  }
+  auto stage = [&](int t, int par) {
+    const float* row = qkv + (size_t)t * C;
+    for (int e = tid; e < 2 * DP; e += 256) {
+      const int which = e / DP, d = e % DP;          // 0: k, 1: q
+      kq[par][e] = d < D ? row[(which ? 0 : GD) + kh * D + d] : 0.f;
+    }
+    if (tid < 64) vv[par][tid] = (vs * 64 + tid) < V ? row[2 * GD + h * V + vs * 64 + tid] : 0.f;
+    if (tid == 64) vv[par][64] = gb[(size_t)t * 2 * H + h];
+    if (tid == 65) vv[par][65] = gb[(size_t)t * 2 * H + H + h];
+  };
+  stage(t0, 0);
+  __syncthreads();
+  for (int t = t0; t < t1; t++) {
+    const int par = (t - t0) & 1;
+    const float g = vv[par][64], beta = vv[par][65], val = vv[par][lane];
+    float kr[DPW];
+    float pk = 0.f, pq = 0.f, dkq = 0.f;
+#pragma unroll
+    for (int r = 0; r < DPW; r++) {
+      const float kd = kq[par][wave * DPW + r], qd = kq[par][DP + wave * DPW + r];
+      kr[r] = kd;
+      S[r] *= g;
+      pk += kd * S[r];
+      pq += qd * S[r];
+      dkq += kd * qd;
+    }
+    red[par][wave][0][lane] = pk;
+    red[par][wave][1][lane] = pq;
+    if (lane == 0) redkq[par][wave] = dkq;
+    if (t + 1 < t1) stage(t + 1, par ^ 1);
+    __syncthreads();
+    const float kS = (red[par][0][0][lane] + red[par][1][0][lane]) + (red[par][2][0][lane] + red[par][3][0][lane]);
+    const float qS = (red[par][0][1][lane] + red[par][1][1][lane]) + (red[par][2][1][lane] + red[par][3][1][lane]);
+    const float kdq = (redkq[par][0] + redkq[par][1]) + (redkq[par][2] + redkq[par][3]);
+    const float u = beta * (val - kS);
+#pragma unroll
+    for (int r = 0; r < DPW; r++) S[r] += kr[r] * u;
+    if (wave == 0 && col < V) o[((size_t)t * H + h) * V + col] = qS + u * kdq;
+  }
+#pragma unroll
+  for (int r = 0; r < DPW; r++) {
+    const int d = wave * DPW + r;
+    if (d < D && col < V) Sp[(size_t)d * V + col] = S[r];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// latent attention: prep (one workgroup per token)
+template <typename KT>
+__global__ void __launch_bounds__(256) latattn_prep_kernel(ktx_latattn_config c, const float* __restrict__ proj, int64_t ldp, int q_off,
+                                                           int c_off, const float* __restrict__ wn, const double* __restrict__ inv_freq,
+                                                           const int32_t* __restrict__ pos, const int32_t* __restrict__ cache_loc,
+                                                           KT* __restrict__ cache, float* __restrict__ q_out) {
+  extern __shared__ float cs[];            // cos | sin of the rot_dims / 2 angles
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int L = c.kv_rank, R = c.rot_dim, E = L + R, NP = c.rot_dims / 2;
+  const double p = (double)pos[t];
+  for (int i = tid; i < NP; i += 256) {
+    const double a = p * inv_freq[i];
+    cs[i] = (float)cos(a);
+    cs[NP + i] = (float)sin(a);
+  }
+  const float* lat = proj + (size_t)t * ldp + c_off;
+  float s = 0.f;
+  for (int e = tid; e < L; e += 256) s += lat[e] * lat[e];
+  const float r = 1.0f / sqrtf(block_sum256(s, red) / (float)L + c.eps);      // (its barriers also publish cs)
+  KT* row = cache + (size_t)cache_loc[t] * E;
+  for (int e = tid; e < L; e += 256) st_elem(row, e, lat[e] * r * wn[e]);
+  // rotated parts: entry j of a rotated vector; j < rot_dims turns with its partner
+  auto turned = [&](const float* v, int j) -> float {
+    if (j >= 2 * NP) return v[j];
+    const int i = j >> 1;
+    const float a = v[2 * i], bb = v[2 * i + 1];
+    return (j & 1) ? bb * cs[i] + a * cs[NP + i] : a * cs[i] - bb * cs[NP + i];
+  };
+  for (int j = tid; j < R; j += 256) st_elem(row, L + j, turned(lat + L, j));
+  const int D = c.dim;
+  for (int e = tid; e < c.heads * R; e += 256) {
+    const int h = e / R, j = e % R;
+    q_out[((size_t)t * c.heads + h) * E + L + j] = turned(proj + (size_t)t * ldp + q_off + (size_t)h * (D + R) + D, j);
+  }
+}
+
+// attention of ONE token (blockIdx.x) x a group of HG heads (blockIdx.y) x one key range (blockIdx.z) on the vector ALUs: tiles of
+// KTN <= 64 keys staged in LDS as fp32; scores thread = (head, key); running maximum / sum per head by wavefronts; outputs thread =
+// (head, latent entry) in registers.
+constexpr int LA_NACC = 32;
+template <typename KT, typename OT>
+__global__ void __launch_bounds__(256) latattn_fwd_kernel(ktx_latattn_config c, int T, int HG, int KTN, const float* __restrict__ q,
+                                                          const KT* __restrict__ cache, const int32_t* __restrict__ tok_req,
+                                                          const int32_t* __restrict__ pos, const int32_t* __restrict__ page_indptr,
+                                                          const int32_t* __restrict__ page_indices, const float* __restrict__ sink,
+                                                          int nsplit, float* __restrict__ scratch, OT* __restrict__ out) {
+  extern __shared__ float lds[];
+  const int L = c.kv_rank, E = L + c.rot_dim, EP = E + 1;
+  float* qs = lds;                         // [HG][E]
+  float* kt = qs + (size_t)HG * E;         // [KTN][EP]
+  float* sc = kt + (size_t)KTN * EP;       // [HG][KTN]
+  float* mrow = sc + (size_t)HG * KTN;     // [HG] running maximum
+  float* lrow = mrow + HG;                 // [HG] running sum
+  float* crow = lrow + HG;                 // [HG] correction of this tile
+  int* rowidx = reinterpret_cast<int*>(crow + HG);   // [KTN]
+  const int t = blockIdx.x, h0 = blockIdx.y * HG, z = blockIdx.z;
+  const int nh = min(HG, c.heads - h0);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int p = pos[t], b = tok_req[t];
+  const int jlo = c.window > 0 ? max(0, p - c.window + 1) : 0, jhi = p + 1;
+  const int per = (jhi - jlo + nsplit - 1) / nsplit;
+  const int j0 = jlo + z * per, j1 = min(jhi, j0 + per);
+  for (int e = tid; e < nh * E; e += 256) qs[e] = q[((size_t)t * c.heads + h0) * E + e];
+  for (int h = tid; h < HG; h += 256) {
+    mrow[h] = -INFINITY;
+    lrow[h] = 0.f;
+  }
+  float acc[LA_NACC];
+#pragma unroll
+  for (int i = 0; i < LA_NACC; i++) acc[i] = 0.f;
+  const int nout = nh * L;
+  const int32_t* pages = page_indices + page_indptr[b];
+  for (int jt = j0; jt < j1; jt += KTN) {
+    const int nk = min(KTN, j1 - jt);
+    __syncthreads();
+    if (tid < nk) {
+      const int j = jt + tid;
+      rowidx[tid] = pages[j / c.page_size] * c.page_size + j % c.page_size;
+    }
+    __syncthreads();
+    for (int e = tid; e < nk * E; e += 256) {
+      const int j = e / E, d = e % E;
+      kt[(size_t)j * EP + d] = ld_elem(cache, (size_t)rowidx[j] * E + d);
+    }
+    __syncthreads();
+    for (int e = tid; e < nh * KTN; e += 256) {
+      const int h = e / KTN, j = e % KTN;
+      if (j < nk) {
+        const float* qh = qs + (size_t)h * E;
+        const float* kj = kt + (size_t)j * EP;
+        float s = 0.f;
+        for (int d = 0; d < E; d++) s += qh[d] * kj[d];
+        sc[(size_t)h * KTN + j] = s * c.scale;
+      }
+    }
+    __syncthreads();
+    for (int h = wave; h < nh; h += 4) {
+      const float s = lane < nk ? sc[(size_t)h * KTN + lane] : -INFINITY;
+      const float mo = mrow[h];
+      const float mn = fmaxf(mo, wave_max(s));
+      const float w = lane < nk ? expf(s - mn) : 0.f;
+      const float sum = wave_sum(w);
+      if (lane < nk) sc[(size_t)h * KTN + lane] = w;
+      if (lane == 0) {
+        const float cr = mo == -INFINITY ? 0.f : expf(mo - mn);
+        crow[h] = cr;
+        mrow[h] = mn;
+        lrow[h] = lrow[h] * cr + sum;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < LA_NACC; i++) {
+      const int e = tid + i * 256;
+      if (e < nout) {
+        const int h = e / L, l = e % L;
+        float a = acc[i] * crow[h];
+        const float* w = sc + (size_t)h * KTN;
+        for (int j = 0; j < nk; j++) a += w[j] * kt[(size_t)j * EP + l];
+        acc[i] = a;
+      }
+    }
+  }
+  __syncthreads();
+  if (nsplit == 1) {
+#pragma unroll
+    for (int i = 0; i < LA_NACC; i++) {
+      const int e = tid + i * 256;
+      if (e < nout) {
+        const int h = e / L, l = e % L;
+        const float sk = sink[h0 + h], m = mrow[h];
+        const float M = fmaxf(m, sk);
+        const float f = m == -INFINITY ? 0.f : expf(m - M);
+        st_elem(out, ((size_t)t * c.heads + h0 + h) * L + l, acc[i] * f / (lrow[h] * f + expf(sk - M)));
+      }
+    }
+    return;
+  }
+  float* part = scratch + (((size_t)z * T + t) * c.heads + h0) * (L + 2);
+#pragma unroll
+  for (int i = 0; i < LA_NACC; i++) {
+    const int e = tid + i * 256;
+    if (e < nout) part[(size_t)(e / L) * (L + 2) + e % L] = acc[i];
+  }
+  for (int h = tid; h < nh; h += 256) {
+    part[(size_t)h * (L + 2) + L] = mrow[h];
+    part[(size_t)h * (L + 2) + L + 1] = lrow[h];
+  }
+}
+
+// merge the key ranges of one (token, head): thread = latent entry
+template <typename OT>
+__global__ void __launch_bounds__(256) latattn_merge_kernel(int T, int H, int L, int nsplit, const float* __restrict__ scratch,
+                                                            const float* __restrict__ sink, OT* __restrict__ out) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const float sk = sink[h];
+  float M = sk;
+  for (int z = 0; z < nsplit; z++) M = fmaxf(M, scratch[(((size_t)z * T + t) * H + h) * (L + 2) + L]);
+  float den = expf(sk - M);
+  for (int z = 0; z < nsplit; z++) {
+    const float* part = scratch + (((size_t)z * T + t) * H + h) * (L + 2);
+    if (part[L] != -INFINITY) den += part[L + 1] * expf(part[L] - M);
+  }
+  for (int l = threadIdx.x; l < L; l += 256) {
+    float a = 0.f;
+    for (int z = 0; z < nsplit; z++) {
+      const float* part = scratch + (((size_t)z * T + t) * H + h) * (L + 2);
+      if (part[L] != -INFINITY) a += part[l] * expf(part[L] - M);
+    }
+    st_elem(out, ((size_t)t * H + h) * L + l, a / den);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// router: one wavefront per token; lane holds experts lane, lane + 64, ... (E <= 64 * RE)
+constexpr int MOE_RE = 16;
+__global__ void __launch_bounds__(256) moe_route_kernel(int T, int E, int top, float scale, float sum_eps,
+                                                        const float* __restrict__ logits, int64_t ldl, int32_t* __restrict__ idx,
+                                                        float* __restrict__ wts) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= T) return;
+  float s[MOE_RE];
+#pragma unroll
+  for (int i = 0; i < MOE_RE; i++) {
+    const int e = lane + i * 64;
+    s[i] = e < E ? sigmoid_f32(logits[(size_t)t * ldl + e]) : -1.f;
+  }
+  float sum = 0.f, mine = 0.f;      // lane k keeps the k-th choice's score
+  int mine_e = 0;
+  for (int k = 0; k < top; k++) {
+    float bv = -1.f;
+    int be = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < MOE_RE; i++) {
+      const int e = lane + i * 64;
+      if (s[i] > bv) {
+        bv = s[i];
+        be = e;
+      }
+    }
+    for (int off = 32; off; off >>= 1) {
+      const float ov = __shfl_xor(bv, off);
+      const int oe = __shfl_xor(be, off);
+      if (ov > bv || (ov == bv && oe < be)) {
+        bv = ov;
+        be = oe;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < MOE_RE; i++)
+      if (lane + i * 64 == be) s[i] = -1.f;
+    sum += bv;
+    if ((k & 63) == lane) {
+      mine = bv;
+      mine_e = be;
+    }
+    if ((k & 63) == 63 || k == top - 1) {      // flush up to 64 choices
+      const int base = k & ~63;
+      if (base + lane <= k) {
+        idx[(size_t)t * top + base + lane] = mine_e;
+        wts[(size_t)t * top + base + lane] = mine;     // normalised below
+      }
+    }
+  }
+  const float f = scale / (sum + sum_eps);
+  for (int k = lane; k < top; k += 64) wts[(size_t)t * top + k] *= f;
+}
+
+// one workgroup sorts the pairs by expert (counting sort in LDS) and lays the row tiles out
+__global__ void __launch_bounds__(1024) moe_plan_kernel(int pairs, int E, int top, int tile_m, const int32_t* __restrict__ idx,
+                                                        int32_t* __restrict__ group_off, int32_t* __restrict__ sorted_tok,
+                                                        int32_t* __restrict__ pair_pos, int32_t* __restrict__ tile_group,
+                                                        int32_t* __restrict__ tile_row0, int32_t* __restrict__ num_tiles) {
+  extern __shared__ int32_t pl[];          // counts [E] | offsets [E + 1] | cursor [E]
+  int32_t* cnt = pl;
+  int32_t* off = pl + E;
+  int32_t* cur = off + E + 1;
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += 1024) cnt[e] = cur[e] = 0;
+  __syncthreads();
+  for (int i = tid; i < pairs; i += 1024) atomicAdd(&cnt[idx[i]], 1);
+  __syncthreads();
+  if (tid == 0) {
+    int at = 0, nt = 0;
+    for (int e = 0; e < E; e++) {
+      off[e] = at;
+      for (int r = 0; r < cnt[e]; r += tile_m) {
+        tile_group[nt] = e;
+        tile_row0[nt] = at + r;
+        nt++;
+      }
+      at += cnt[e];
+    }
+    off[E] = at;
+    num_tiles[0] = nt;
+  }
+  __syncthreads();
+  for (int e = tid; e <= E; e += 1024) group_off[e] = off[e];
+  for (int i = tid; i < pairs; i += 1024) {
+    const int e = idx[i];
+    const int p = off[e] + atomicAdd(&cur[e], 1);
+    sorted_tok[p] = i / top;
+    pair_pos[i] = p;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// grouped GEMM: the 64 x 64 x 32 tile of the dense kernel; a tile belongs to one group (its weights), rows may be gathered
+template <typename AT, typename CT>
+__device__ __forceinline__ void gg_stage_rows(CT* dst, const AT* __restrict__ src, int64_t ld, const int32_t* __restrict__ rows,
+                                              int row0, int row_end, int k0, int K, bool vec) {
+  const int r = threadIdx.x >> 2, seg = (threadIdx.x & 3) * 8;
+  const int gr = row0 + r;
+  CT* d = dst + r * GemmTraits<CT>::LDS_LD + seg;
+  const bool live = gr < row_end;
+  const size_t srow = live ? (size_t)(rows ? rows[gr] : gr) : 0;
+  if (live && vec && k0 + seg + 8 <= K) {
+    const AT* s = src + srow * ld + k0 + seg;
+    if constexpr (sizeof(AT) == 2 && sizeof(CT) == 2) {
+      *reinterpret_cast<uint4*>(d) = *reinterpret_cast<const uint4*>(s);
+    } else if constexpr (sizeof(AT) == 4 && sizeof(CT) == 2) {
+      const float4 a = *reinterpret_cast<const float4*>(s), b = *reinterpret_cast<const float4*>(s + 4);
+      uint4 o;
+      o.x = ktx_pk_bf16(a.x, a.y); o.y = ktx_pk_bf16(a.z, a.w); o.z = ktx_pk_bf16(b.x, b.y); o.w = ktx_pk_bf16(b.z, b.w);
+      *reinterpret_cast<uint4*>(d) = o;
+    } else {
+      const float4 a = *reinterpret_cast<const float4*>(s), b = *reinterpret_cast<const float4*>(s + 4);
+      d[0] = a.x; d[1] = a.y; d[2] = a.z; d[3] = a.w; d[4] = b.x; d[5] = b.y; d[6] = b.z; d[7] = b.w;
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int k = k0 + seg + i;
+    float v = 0.f;
+    if (live && k < K) v = ld_elem(src, srow * ld + k);
+    if constexpr (sizeof(CT) == 2) d[i] = to_bf16_rne(v);
+    else d[i] = v;
+  }
+}
+
+template <typename AT, typename CT, typename YT>
+__global__ void __launch_bounds__(256) grouped_gemm_kernel(int M, int N, int K, const AT* __restrict__ A, int64_t lda, int64_t a_goff,
+                                                           const int32_t* __restrict__ a_rows, const CT* __restrict__ W,
+                                                           YT* __restrict__ Y, int64_t ldy, int64_t y_goff,
+                                                           const int32_t* __restrict__ group_off, const int32_t* __restrict__ tile_group,
+                                                           const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ num_tiles,
+                                                           bool vec_a, bool vec_w) {
+  constexpr int LD = GemmTraits<CT>::LDS_LD;
+  __shared__ __attribute__((aligned(16))) CT As[64 * LD];
+  __shared__ __attribute__((aligned(16))) CT Ws[64 * LD];
+  int g, m0, m_end;
+  if (group_off) {
+    if ((int)blockIdx.y >= num_tiles[0]) return;
+    g = tile_group[blockIdx.y];
+    m0 = tile_row0[blockIdx.y];
+    m_end = group_off[g + 1];
+  } else {
+    g = blockIdx.z;
+    m0 = blockIdx.y * 64;
+    m_end = M;
+    A += a_goff * g;
+    Y += y_goff * g;
+  }
+  const CT* Wg = W + (size_t)g * N * K;
+  const int n0 = blockIdx.x * 64;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+  const int l16 = lane & 15, lq = lane >> 4;
+  v4f acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    __syncthreads();
+    gg_stage_rows<AT, CT>(As, A, lda, a_rows, m0, m_end, k0, K, vec_a);
+    gemm_stage<CT, CT>(Ws, Wg, (int64_t)K, n0, N, k0, K, vec_w);
+    __syncthreads();
+    if constexpr (sizeof(CT) == 2) {
+      sq_v8bf af[2], bf[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        af[i] = *reinterpret_cast<const sq_v8bf*>(As + (wm + i * 16 + l16) * LD + lq * 8);
+        bf[i] = *reinterpret_cast<const sq_v8bf*>(Ws + (wn + i * 16 + l16) * LD + lq * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < 32; kk += 4) {
+        float af[2], bf[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+          af[i] = As[(wm + i * 16 + l16) * LD + kk + lq];
+          bf[i] = Ws[(wn + i * 16 + l16) * LD + kk + lq];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int m = m0 + wm + i * 16 + lq * 4 + r, n = n0 + wn + j * 16 + l16;
+        if (m < m_end && n < N) st_elem(Y, (size_t)m * ldy + n, acc[i][j][r]);
+      }
+}
+
+int dtype_ok(int d) { return d == KTX_SEQ_F32 || d == KTX_SEQ_BF16; }
+
+}  // namespace
+
+extern "C" {
+
+int ktx_rows_add(int T, int W, float* d_x, const float* d_x0, const float* d_vec, ktx_stream_t stream) {
+  KTX_REQUIRE(T >= 0 && W > 0 && d_x, "ktx_rows_add: T >= 0, W > 0, x");
+  if (T == 0 || (!d_x0 && !d_vec)) return 0;
+  const size_t n = (size_t)T * W;
+  rows_add_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(n, W, d_x, d_x0, d_vec);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_layer_norm(int T, int W, const float* d_x, const float* d_w, const float* d_b, float eps, const int32_t* d_rows, void* d_out,
+                   int out_dtype, ktx_stream_t stream) {
+  KTX_REQUIRE(T >= 0 && W > 0 && d_x && d_w && d_out && dtype_ok(out_dtype), "ktx_layer_norm: arguments");
+  if (T == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == KTX_SEQ_F32) layer_norm_kernel<float><<<T, 256, 0, st>>>(W, d_x, d_w, d_b, eps, d_rows, (float*)d_out);
+  else layer_norm_kernel<bf16_t><<<T, 256, 0, st>>>(W, d_x, d_w, d_b, eps, d_rows, (bf16_t*)d_out);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_gated_norm_add(int T, int W, const float* d_y, int64_t ldy, const float* d_ybias, const float* d_ey, const int32_t* d_pair_pos,
+                       const float* d_topk_w, int top, const float* d_gl, int64_t ldg, const float* d_gbias, const float* d_wn,
+                       const float* d_bn, float eps, float* d_x, ktx_stream_t stream) {
+  KTX_REQUIRE(T >= 0 && W > 0 && d_wn && d_x && (d_y || d_ey), "ktx_gated_norm_add: arguments");
+  KTX_REQUIRE(!d_ey || (d_pair_pos && d_topk_w && top > 0), "ktx_gated_norm_add: the gathered term needs pair_pos, topk_w and top");
+  KTX_REQUIRE((size_t)W * 4 <= 64 * 1024, "ktx_gated_norm_add: rows up to 16384 entries");
+  if (T == 0) return 0;
+  gated_norm_add_kernel<<<T, 256, (size_t)W * 4, (hipStream_t)stream>>>(W, d_y, ldy, d_ybias, d_ey, d_pair_pos, d_topk_w, top, d_gl, ldg,
+                                                                          d_gbias, d_wn, d_bn, eps, d_x);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_poly_norm(int T, int F, const float* d_z, int64_t ldz, const float* d_bias, const float* d_coef, float eps, void* d_out,
+                  int out_dtype, ktx_stream_t stream) {
+  KTX_REQUIRE(T >= 0 && F > 0 && d_z && d_coef && d_out && dtype_ok(out_dtype) && ldz >= F, "ktx_poly_norm: arguments");
+  if (T == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == KTX_SEQ_F32) poly_norm_kernel<float><<<T, 256, 0, st>>>(F, d_z, ldz, d_bias, d_coef, eps, (float*)d_out);
+  else poly_norm_kernel<bf16_t><<<T, 256, 0, st>>>(F, d_z, ldz, d_bias, d_coef, eps, (bf16_t*)d_out);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_silu_mul_rows(int R, int F, const float* d_in, int64_t ldi, void* d_out, int out_dtype, ktx_stream_t stream) {
+  KTX_REQUIRE(R >= 0 && F > 0 && d_in && d_out && dtype_ok(out_dtype) && ldi >= 2 * (int64_t)F, "ktx_silu_mul_rows: arguments");
+  if (R == 0) return 0;
+  const size_t n = (size_t)R * F;
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == KTX_SEQ_F32) silu_mul_rows_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(n, F, d_in, ldi, (float*)d_out);
+  else silu_mul_rows_kernel<bf16_t><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(n, F, d_in, ldi, (bf16_t*)d_out);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_head_gate_norm(int T, int heads, int vdim, float eps, const float* d_o, const float* d_gate, int64_t ldg, const float* d_w,
+                       int w_per_head, int act, void* d_out, int out_dtype, ktx_stream_t stream) {
+  KTX_REQUIRE(T >= 0 && heads > 0 && vdim > 0 && d_o && d_gate && d_w && d_out && dtype_ok(out_dtype), "ktx_head_gate_norm: arguments");
+  if (T == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == KTX_SEQ_F32)
+    head_gate_norm_kernel<float><<<T, 256, 0, st>>>(heads, vdim, eps, d_o, d_gate, ldg, d_w, w_per_head, act, (float*)d_out);
+  else
+    head_gate_norm_kernel<bf16_t><<<T, 256, 0, st>>>(heads, vdim, eps, d_o, d_gate, ldg, d_w, w_per_head, act, (bf16_t*)d_out);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+static int delta_check(const ktx_delta_config* c, const char* who) {
+  if (!c || c->heads <= 0 || c->kv_heads <= 0 || c->heads % c->kv_heads || c->dim <= 0 || c->vdim <= 0 || c->taps < 1)
+    return ktx_fail(std::string(who) + ": heads % kv_heads == 0, dim, vdim > 0, taps >= 1");
+  return 0;
+}
+
+int ktx_delta_prep(const ktx_delta_config* cfg, int B, int T, const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_slot,
+                   const int32_t* d_tok_req, const float* d_proj, int64_t ldp, int q_off, int k_off, int v_off, int b_off, int a_off,
+                   const float* d_taps, const float* d_A_log, const float* d_dt_bias, float* d_conv_state, float* d_qkv, float* d_gb,
+                   ktx_stream_t stream) {
+  if (delta_check(cfg, "ktx_delta_prep")) return -1;
+  KTX_REQUIRE(B >= 0 && T >= 0 && d_q_indptr && d_pos0 && d_slot && d_tok_req && d_proj && d_taps && d_A_log && d_dt_bias && d_qkv && d_gb,
+              "ktx_delta_prep: null pointer");
+  KTX_REQUIRE(cfg->taps == 1 || d_conv_state, "ktx_delta_prep: a convolution over time needs its state");
+  if (T == 0 || B == 0) return 0;
+  const int C = 2 * cfg->kv_heads * cfg->dim + cfg->heads * cfg->vdim;
+  const size_t lds = (size_t)C * 4;
+  KTX_REQUIRE(lds <= 128 * 1024, "ktx_delta_prep: q | k | v of one token must fit 128 KB of LDS");
+  hipStream_t st = (hipStream_t)stream;
+  KTX_HIP(ktx_set_max_lds((const void*)delta_prep_kernel, 128 * 1024));
+  delta_prep_kernel<<<T, 256, lds, st>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_tok_req, d_proj, ldp, q_off, k_off, v_off, b_off, a_off,
+                                         d_taps, d_A_log, d_dt_bias, d_conv_state, d_qkv, d_gb);
+  KTX_HIP(hipGetLastError());
+  if (cfg->taps > 1) {
+    delta_conv_update_kernel<<<dim3((C + 255) / 256, B), 256, 0, st>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_proj, ldp, q_off, k_off, v_off,
+                                                                       d_conv_state);
+    KTX_HIP(hipGetLastError());
+  }
+  return 0;
+}
+
+int ktx_delta_forward(const ktx_delta_config* cfg, int B, const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_slot,
+                      const float* d_qkv, const float* d_gb, float* d_S, float* d_o, ktx_stream_t stream) {
+  if (delta_check(cfg, "ktx_delta_forward")) return -1;
+  KTX_REQUIRE(B >= 0 && d_q_indptr && d_pos0 && d_slot && d_qkv && d_gb && d_S && d_o, "ktx_delta_forward: null pointer");
+  KTX_REQUIRE(cfg->dim <= 256, "ktx_delta_forward: dim <= 256");
+  if (B == 0) return 0;
+  const unsigned blocks = (unsigned)B * cfg->heads * ((cfg->vdim + 63) / 64);
+  hipStream_t st = (hipStream_t)stream;
+  const int dpw = (cfg->dim + 3) / 4;
+#define KTX_DL_GO(DPW) delta_fwd_kernel<DPW><<<blocks, 256, 0, st>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_qkv, d_gb, d_S, d_o)
+  if (dpw <= 4) KTX_DL_GO(4);
+  else if (dpw <= 8) KTX_DL_GO(8);
+  else if (dpw <= 16) KTX_DL_GO(16);
+  else if (dpw <= 32) KTX_DL_GO(32);
+  else KTX_DL_GO(64);
+#undef KTX_DL_GO
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+static int latattn_check(const ktx_latattn_config* c, const char* who) {
+  if (!c || c->heads <= 0 || c->dim <= 0 || c->rot_dim < 0 || c->vdim <= 0 || c->kv_rank <= 0 || c->rot_dims < 0 || (c->rot_dims & 1) ||
+      c->rot_dims > c->rot_dim || c->page_size <= 0 || !dtype_ok(c->cache_dtype))
+    return ktx_fail(std::string(who) + ": sizes > 0, rot_dims even and <= rot_dim, a known cache type");
+  return 0;
+}
+
+int ktx_latattn_prep(const ktx_latattn_config* cfg, int T, const float* d_proj, int64_t ldp, int q_off, int c_off, const float* d_wn,
+                     const double* d_inv_freq, const int32_t* d_pos, const int32_t* d_cache_loc, void* d_cache, float* d_q_out,
+                     ktx_stream_t stream) {
+  if (latattn_check(cfg, "ktx_latattn_prep")) return -1;
+  KTX_REQUIRE(T >= 0 && d_proj && d_wn && (d_inv_freq || cfg->rot_dims == 0) && d_pos && d_cache_loc && d_cache && d_q_out,
+              "ktx_latattn_prep: null pointer");
+  if (T == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  const size_t lds = (size_t)std::max(cfg->rot_dims, 2) * 4;
+  if (cfg->cache_dtype == KTX_SEQ_F32)
+    latattn_prep_kernel<float><<<T, 256, lds, st>>>(*cfg, d_proj, ldp, q_off, c_off, d_wn, d_inv_freq, d_pos, d_cache_loc, (float*)d_cache, d_q_out);
+  else
+    latattn_prep_kernel<bf16_t><<<T, 256, lds, st>>>(*cfg, d_proj, ldp, q_off, c_off, d_wn, d_inv_freq, d_pos, d_cache_loc, (bf16_t*)d_cache, d_q_out);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_latattn_forward(const ktx_latattn_config* cfg, int T, const float* d_q, const void* d_cache, const int32_t* d_tok_req,
+                        const int32_t* d_pos, const int32_t* d_page_indptr, const int32_t* d_page_indices, const float* d_sink,
+                        int nsplit, float* d_scratch, void* d_out, int out_dtype, ktx_stream_t stream) {
+  if (latattn_check(cfg, "ktx_latattn_forward")) return -1;
+  KTX_REQUIRE(T >= 0 && d_q && d_cache && d_tok_req && d_pos && d_page_indptr && d_page_indices && d_sink && d_out && dtype_ok(out_dtype),
+              "ktx_latattn_forward: null pointer");
+  KTX_REQUIRE(nsplit >= 1 && nsplit <= 65535 && (nsplit == 1 || d_scratch), "ktx_latattn_forward: nsplit >= 1, scratch when > 1");
+  if (T == 0) return 0;
+  const int L = cfg->kv_rank, E = L + cfg->rot_dim;
+  KTX_REQUIRE(L <= 256 * LA_NACC, "ktx_latattn_forward: kv_rank <= 8192");
+  // heads per workgroup: outputs fit the registers, queries + one key tile fit the LDS
+  const size_t budget = 96 * 1024;
+  int HG = std::min(cfg->heads, std::max(1, 256 * LA_NACC / L));
+  int KTN = 64;
+  auto lds_of = [&](int hg, int ktn) { return ((size_t)hg * E + (size_t)ktn * (E + 1) + (size_t)hg * ktn + 3 * (size_t)hg + ktn) * 4; };
+  while (KTN > 8 && lds_of(1, KTN) > budget) KTN /= 2;
+  while (HG > 1 && lds_of(HG, KTN) > budget) HG = (HG + 1) / 2;
+  KTX_REQUIRE(lds_of(HG, KTN) <= 150 * 1024, "ktx_latattn_forward: one head's query and 8 keys do not fit the LDS");
+  const size_t lds = lds_of(HG, KTN);
+  const dim3 grid(T, (cfg->heads + HG - 1) / HG, nsplit);
+  hipStream_t st = (hipStream_t)stream;
+#define KTX_LA_GO(KT, OT)                                                                                                     \
+  do {                                                                                                                        \
+    KTX_HIP(ktx_set_max_lds((const void*)latattn_fwd_kernel<KT, OT>, 150 * 1024));                                            \
+    latattn_fwd_kernel<KT, OT><<<grid, 256, lds, st>>>(*cfg, T, HG, KTN, d_q, (const KT*)d_cache, d_tok_req, d_pos, d_page_indptr, \
+                                                       d_page_indices, d_sink, nsplit, d_scratch, (OT*)d_out);               \
+  } while (0)
+  if (cfg->cache_dtype == KTX_SEQ_F32) {
+    if (out_dtype == KTX_SEQ_F32) KTX_LA_GO(float, float);
+    else KTX_LA_GO(float, bf16_t);
+  } else {
+    if (out_dtype == KTX_SEQ_F32) KTX_LA_GO(bf16_t, float);
+    else KTX_LA_GO(bf16_t, bf16_t);
+  }
+#undef KTX_LA_GO
+  KTX_HIP(hipGetLastError());
+  if (nsplit > 1) {
+    const dim3 mg(T, cfg->heads);
+    if (out_dtype == KTX_SEQ_F32) latattn_merge_kernel<float><<<mg, 256, 0, st>>>(T, cfg->heads, L, nsplit, d_scratch, d_sink, (float*)d_out);
+    else latattn_merge_kernel<bf16_t><<<mg, 256, 0, st>>>(T, cfg->heads, L, nsplit, d_scratch, d_sink, (bf16_t*)d_out);
+    KTX_HIP(hipGetLastError());
+  }
+  return 0;
+}
+
+int ktx_moe_route(int T, int E, int top, float scale, float sum_eps, const float* d_logits, int64_t ldl, int32_t* d_topk_idx,
+                  float* d_topk_w, ktx_stream_t stream) {
+  KTX_REQUIRE(T >= 0 && E > 0 && top > 0 && top <= E && E <= 64 * MOE_RE && d_logits && d_topk_idx && d_topk_w && ldl >= E,
+              "ktx_moe_route: 0 < top <= experts <= 1024");
+  if (T == 0) return 0;
+  moe_route_kernel<<<(T + 3) / 4, 256, 0, (hipStream_t)stream>>>(T, E, top, scale, sum_eps, d_logits, ldl, d_topk_idx, d_topk_w);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_moe_plan(int T, int E, int top, int tile_m, const int32_t* d_topk_idx, int32_t* d_group_off, int32_t* d_sorted_tok,
+                 int32_t* d_pair_pos, int32_t* d_tile_group, int32_t* d_tile_row0, int32_t* d_num_tiles, ktx_stream_t stream) {
+  KTX_REQUIRE(T >= 0 && E > 0 && E <= 4096 && top > 0 && tile_m > 0 && d_topk_idx && d_group_off && d_sorted_tok && d_pair_pos &&
+                  d_tile_group && d_tile_row0 && d_num_tiles,
+              "ktx_moe_plan: arguments");
+  moe_plan_kernel<<<1, 1024, (size_t)(3 * E + 1) * 4, (hipStream_t)stream>>>(T * top, E, top, tile_m, d_topk_idx, d_group_off, d_sorted_tok,
+                                                                              d_pair_pos, d_tile_group, d_tile_row0, d_num_tiles);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_grouped_gemm(int G, int M, int N, int K, const void* d_A, int a_dtype, int64_t lda, int64_t a_goff, const int32_t* d_a_rows,
+                     const void* d_W, int w_dtype, void* d_Y, int y_dtype, int64_t ldy, int64_t y_goff, const int32_t* d_group_off,
+                     const int32_t* d_tile_group, const int32_t* d_tile_row0, const int32_t* d_num_tiles, int max_tiles,
+                     ktx_stream_t stream) {
+  KTX_REQUIRE(G > 0 && M >= 0 && N > 0 && K > 0 && d_A && d_W && d_Y, "ktx_grouped_gemm: G, N, K > 0, pointers");
+  KTX_REQUIRE(dtype_ok(a_dtype) && dtype_ok(w_dtype) && dtype_ok(y_dtype), "ktx_grouped_gemm: unknown element type");
+  KTX_REQUIRE(!(w_dtype == KTX_SEQ_F32 && (a_dtype != KTX_SEQ_F32 || y_dtype != KTX_SEQ_F32)),
+              "ktx_grouped_gemm: an fp32 product takes and writes fp32");
+  const bool ragged = d_group_off != nullptr;
+  KTX_REQUIRE(!ragged || (d_tile_group && d_tile_row0 && d_num_tiles && max_tiles >= 0), "ktx_grouped_gemm: the ragged form needs its tiles");
+  KTX_REQUIRE(ragged || (G <= 65535 && !d_a_rows), "ktx_grouped_gemm: the uniform form takes up to 65535 groups and no gather");
+  const int ytiles = ragged ? max_tiles : (M + 63) / 64;
+  if (ytiles == 0) return 0;
+  KTX_REQUIRE(ytiles <= 65535, "ktx_grouped_gemm: too many row tiles");
+  const dim3 grid((N + 63) / 64, ytiles, ragged ? 1 : G);
+  const size_t asz = a_dtype == KTX_SEQ_F32 ? 4 : 2, wsz = w_dtype == KTX_SEQ_F32 ? 4 : 2;
+  const bool vec_a = aligned16(d_A) && (lda * asz) % 16 == 0 && ((size_t)a_goff * asz) % 16 == 0 && K % 8 == 0;
+  const bool vec_w = aligned16(d_W) && ((size_t)K * wsz) % 16 == 0 && K % 8 == 0 && ((size_t)N * K * wsz) % 16 == 0;
+  hipStream_t st = (hipStream_t)stream;
+#define KTX_GG_GO(AT, CT, YT)                                                                                                  \
+  grouped_gemm_kernel<AT, CT, YT><<<grid, 256, 0, st>>>(M, N, K, (const AT*)d_A, lda, a_goff, d_a_rows, (const CT*)d_W, (YT*)d_Y, ldy, \
+                                                        y_goff, d_group_off, d_tile_group, d_tile_row0, d_num_tiles, vec_a, vec_w)
+  if (w_dtype == KTX_SEQ_BF16) {
+    if (a_dtype == KTX_SEQ_F32 && y_dtype == KTX_SEQ_F32) KTX_GG_GO(float, bf16_t, float);
+    else if (a_dtype == KTX_SEQ_F32) KTX_GG_GO(float, bf16_t, bf16_t);
+    else if (y_dtype == KTX_SEQ_F32) KTX_GG_GO(bf16_t, bf16_t, float);
+    else KTX_GG_GO(bf16_t, bf16_t, bf16_t);
+  } else {
+    KTX_GG_GO(float, float, float);
+  }
+#undef KTX_GG_GO
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // extern "C"

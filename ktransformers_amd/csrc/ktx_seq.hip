@@ -14,34 +14,9 @@
 
 #include <algorithm>
 
-typedef __bf16 sq_v8bf __attribute__((ext_vector_type(8)));
-
 namespace {
 
-__device__ __forceinline__ float ld_elem(const float* p, size_t i) { return p[i]; }
-__device__ __forceinline__ float ld_elem(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }
-__device__ __forceinline__ void st_elem(float* p, size_t i, float v) { p[i] = v; }
-__device__ __forceinline__ void st_elem(bf16_t* p, size_t i, float v) { p[i] = (bf16_t)(ktx_pk_bf16(v, 0.f) & 0xffffu); }
-__device__ __forceinline__ bf16_t to_bf16_rne(float v) { return (bf16_t)(ktx_pk_bf16(v, 0.f) & 0xffffu); }
-
-// sum over the 256 threads of a workgroup; `red` = 4 floats of LDS; every thread gets the result
-__device__ __forceinline__ float block_sum256(float v, float* red) {
-  v = wave_sum(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  return ((red[0] + red[1]) + red[2]) + red[3];
-}
-
-__device__ __forceinline__ float sigmoid_f32(float z) { return 1.0f / (1.0f + expf(-z)); }
-// v_exp_f32 + v_rcp_f32 (about 1 ulp each): the matrix-core attention kernel, whose operands are bf16 anyway
-__device__ __forceinline__ float sigmoid_fast(float z) {
-  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z));
-}
-__device__ __forceinline__ float gelu_tanh_f32(float z) {
-  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-}
-__device__ __forceinline__ float log_sigmoid_f32(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+#include "ktx_seq_dev.inc"
 
 // ---------------------------------------------------------------------------------------------------------------------
 // embedding + sinusoidal positions
@@ -52,6 +27,10 @@ __global__ void __launch_bounds__(256) embed_sinpos_kernel(int width, int vocab,
   const int t = blockIdx.x;
   int id = tok[t];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  if (!inv_freq) {      // a plain table row (positions enter elsewhere)
+    for (int e = threadIdx.x; e < width; e += 256) x[(size_t)t * width + e] = ld_elem(embed, (size_t)id * width + e);
+    return;
+  }
   const double p = (double)pos[t];
   for (int e = threadIdx.x; e < width; e += 256) {
     const double ang = p * inv_freq[e >> 1];
@@ -62,49 +41,6 @@ __global__ void __launch_bounds__(256) embed_sinpos_kernel(int width, int vocab,
 
 // ---------------------------------------------------------------------------------------------------------------------
 // dense GEMM  Y = act(A W^T): 64 x 64 tile, BK = 32, 4 wavefronts of 32 x 32; any shape (edges zero-filled / masked).
-template <typename T>
-struct GemmTraits;
-template <>
-struct GemmTraits<bf16_t> {
-  static constexpr int LDS_LD = 40;   // bf16 elements per tile row: 32 + 8 (16-byte aligned rows, 20-word stride)
-};
-template <>
-struct GemmTraits<float> {
-  static constexpr int LDS_LD = 33;   // odd word stride: the per-lane scalar fragment reads are conflict-free
-};
-
-template <typename AT, typename CT>
-__device__ __forceinline__ void gemm_stage(CT* dst, const AT* __restrict__ src, int64_t ld, int row0, int rows, int k0, int K,
-                                           bool vec) {
-  // thread -> (row = tid / 4, 8 consecutive k)
-  const int r = threadIdx.x >> 2, seg = (threadIdx.x & 3) * 8;
-  const int gr = row0 + r;
-  CT* d = dst + r * GemmTraits<CT>::LDS_LD + seg;
-  if (gr < rows && vec && k0 + seg + 8 <= K) {
-    const AT* s = src + (size_t)gr * ld + k0 + seg;
-    if constexpr (sizeof(AT) == 2 && sizeof(CT) == 2) {
-      *reinterpret_cast<uint4*>(d) = *reinterpret_cast<const uint4*>(s);
-    } else if constexpr (sizeof(AT) == 4 && sizeof(CT) == 2) {
-      const float4 a = *reinterpret_cast<const float4*>(s), b = *reinterpret_cast<const float4*>(s + 4);
-      uint4 o;
-      o.x = ktx_pk_bf16(a.x, a.y); o.y = ktx_pk_bf16(a.z, a.w); o.z = ktx_pk_bf16(b.x, b.y); o.w = ktx_pk_bf16(b.z, b.w);
-      *reinterpret_cast<uint4*>(d) = o;
-    } else {
-      const float4 a = *reinterpret_cast<const float4*>(s), b = *reinterpret_cast<const float4*>(s + 4);
-      d[0] = a.x; d[1] = a.y; d[2] = a.z; d[3] = a.w; d[4] = b.x; d[5] = b.y; d[6] = b.z; d[7] = b.w;
-    }
-    return;
-  }
-#pragma unroll
-  for (int i = 0; i < 8; i++) {
-    const int k = k0 + seg + i;
-    float v = 0.f;
-    if (gr < rows && k < K) v = ld_elem(src, (size_t)gr * ld + k);
-    if constexpr (sizeof(CT) == 2) d[i] = to_bf16_rne(v);
-    else d[i] = v;
-  }
-}
-
 template <typename AT, typename CT, typename YT>
 __global__ void __launch_bounds__(256) dense_gemm_kernel(int M, int N, int K, const AT* __restrict__ A, int64_t lda,
                                                          const CT* __restrict__ W, YT* __restrict__ Y, int64_t ldy, int act,
@@ -1228,7 +1164,7 @@ extern "C" {
 int ktx_embed_sinpos(int T, int width, int vocab, const int32_t* d_tokens, const int32_t* d_pos, const void* d_embed,
                      int embed_dtype, const double* d_inv_freq, float* d_x, ktx_stream_t stream) {
   KTX_REQUIRE(T >= 0 && width > 0 && vocab > 0, "ktx_embed_sinpos: T >= 0, width, vocab > 0");
-  KTX_REQUIRE(d_tokens && d_pos && d_embed && d_inv_freq && d_x, "ktx_embed_sinpos: null pointer");
+  KTX_REQUIRE(d_tokens && d_embed && d_x && (d_pos || !d_inv_freq), "ktx_embed_sinpos: null pointer");
   if (T == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
   if (embed_dtype == KTX_SEQ_BF16)

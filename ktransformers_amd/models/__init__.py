@@ -56,6 +56,17 @@ def _mitotar_cache(config, max_tokens, max_requests, dtype, device):
     return KHybridCache(mitotar_layer_specs(config), max_tokens, max_requests=max_requests, dtype=dtype, device=device)
 
 
+def _pilavik_config(d, dtype):
+    from ktransformers_amd.models.modeling_pilavik import make_pilavik_config
+    return make_pilavik_config(d, dtype)
+
+
+def _pilavik_cache(config, max_tokens, max_requests, dtype, device):
+    from ktransformers_amd.models.custom_cache import KHybridCache
+    from ktransformers_amd.models.modeling_pilavik import pilavik_layer_specs
+    return KHybridCache(pilavik_layer_specs(config), max_tokens, max_requests=max_requests, dtype=dtype, device=device)
+
+
 def _cls(module: str, name: str):
     def get():
         import importlib
@@ -72,6 +83,8 @@ MODEL_REGISTRY = {
                                      "Mixtral-8x7B.yaml", _mixtral_cache),
     "Mitotar": ModelEntry(_mitotar_config, _cls("ktransformers_amd.models.modeling_mitotar", "MitotarForCausalLM"), "Mitotar.yaml",
                           _mitotar_cache, dtypes=(torch.bfloat16, torch.float32)),
+    "Pilavik": ModelEntry(_pilavik_config, _cls("ktransformers_amd.models.modeling_pilavik", "PilavikForCausalLM"), "Pilavik.yaml",
+                          _pilavik_cache, dtypes=(torch.bfloat16, torch.float32)),
 }
 
 

@@ -169,14 +169,19 @@ class ForwardBatch:
 class KHybridCache:
     """Cache and state manager of decoders that mix paged attention with recurrent layers.
 
-    Per attention layer: one paged KEY cache [pages * page_size, kv_heads, dim] (bf16 or fp32) — the design's values are the
-    un-normed keys, so no value cache exists — and fp32 1 / rms(k) per row and key head; per recurrent layer: state slots
-    S [slots, heads, dim, vdim], n [slots, heads, dim], m [slots, heads] in fp32.  A request holds a list of pages (grown as it
-    grows) and one slot from admit() to release(); freed pages and slots go back on LIFO free lists and are handed out again
-    without being cleared: the attention kernels never read past a request's length and the recurrence starts from zero at
-    position 0 whatever the slot holds.
+    Per layer, whatever its spec names:
+      "attn": (kv_heads, dim)  — a paged KEY cache [pages * page_size, kv_heads, dim] (bf16 or fp32) for attention whose values are its
+                                 un-normed keys, plus fp32 1 / rms(k) per row and key head;
+      "latent": width          — a paged cache of latent rows [pages * page_size, width] (bf16 or fp32): what a latent attention keeps
+                                 per token (normed latent + rotated key part);
+      "rec": (heads, dim, vdim)   — fp32 state slots S [slots, heads, dim, vdim], n [slots, heads, dim], m [slots, heads] (mLSTM);
+      "delta": (heads, dim, vdim) — fp32 state slots S alone (delta rule);
+      "conv": (channels, taps)    — fp32 slots [slots, taps - 1, channels]: the inputs a short causal convolution still needs.
+    A layer that runs several times with the same weights (a repeated block) has one spec, and so one cache or state, per run.
+    A request holds a list of pages (grown as it grows) and one slot from admit() to release(); freed pages and slots go back on
+    LIFO free lists and are handed out again without being cleared: the attention kernels never read past a request's length and
+    the recurrences start from zero at position 0 whatever the slot holds.
 
-    layer_specs: per layer {"attn": (kv_heads, dim) | None, "rec": (heads, dim, vdim) | None}.
     plan() turns (request, n new tokens) pairs into a ForwardBatch; the operators append and read through it."""
 
     def __init__(self, layer_specs, max_tokens: int, max_requests: int = 8, page_size: int = 64, dtype=torch.bfloat16,
@@ -189,12 +194,19 @@ class KHybridCache:
         self.num_pages = (int(max_tokens) + self.page_size - 1) // self.page_size + self.max_requests
         self.max_cache_len = self.num_pages * self.page_size
         rows = self.num_pages * self.page_size
-        self.k_caches, self.k_inv, self.S, self.n, self.m = [], [], [], [], []
+        self.k_caches, self.k_inv, self.S, self.n, self.m, self.lat_caches, self.conv = [], [], [], [], [], [], []
         for spec in self.layer_specs:
-            a, r = spec.get("attn"), spec.get("rec")
+            a, r, lat, dl, cv = spec.get("attn"), spec.get("rec"), spec.get("latent"), spec.get("delta"), spec.get("conv")
+            if r and dl:
+                raise ValueError("KHybridCache: a layer run has one recurrent state (\"rec\" or \"delta\")")
             self.k_caches.append(torch.zeros((rows, a[0], a[1]), dtype=dtype, device=self.device) if a else None)
             self.k_inv.append(torch.zeros((rows, a[0]), dtype=torch.float32, device=self.device) if a else None)
+            self.lat_caches.append(torch.zeros((rows, int(lat)), dtype=dtype, device=self.device) if lat else None)
+            self.conv.append(torch.zeros((self.max_requests, cv[1] - 1, cv[0]), dtype=torch.float32, device=self.device)
+                             if cv and cv[1] > 1 else None)
+            r = r or dl
             self.S.append(torch.zeros((self.max_requests, r[0], r[1], r[2]), dtype=torch.float32, device=self.device) if r else None)
+            r = spec.get("rec")
             self.n.append(torch.zeros((self.max_requests, r[0], r[1]), dtype=torch.float32, device=self.device) if r else None)
             self.m.append(torch.zeros((self.max_requests, r[0]), dtype=torch.float32, device=self.device) if r else None)
         self.free_pages = list(range(self.num_pages - 1, -1, -1))
@@ -218,6 +230,10 @@ class KHybridCache:
     def seq_len(self, rid) -> int:
         return self.requests[rid]["len"]
 
+    def state_tensors(self) -> list:
+        """Every per-slot tensor a step advances in place (what a caller saves around runs that must not count)."""
+        return [t for group in (self.S, self.n, self.m, self.conv) for t in group if t is not None]
+
     def live_tokens(self) -> int:
         return sum(r["len"] for r in self.requests.values())
 
@@ -234,6 +250,7 @@ class KHybridCache:
     def _add_slots(self, extra: int) -> None:
         grow = lambda t: None if t is None else torch.cat([t, torch.zeros((extra,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)])
         self.S, self.n, self.m = [grow(t) for t in self.S], [grow(t) for t in self.n], [grow(t) for t in self.m]
+        self.conv = [grow(t) for t in self.conv]
         self.free_slots.extend(range(self.max_requests + extra - 1, self.max_requests - 1, -1))
         self.max_requests += extra
         self.generation += 1
@@ -242,6 +259,7 @@ class KHybridCache:
         rows = extra * self.page_size
         grow = lambda t: None if t is None else torch.cat([t, torch.zeros((rows,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)])
         self.k_caches, self.k_inv = [grow(t) for t in self.k_caches], [grow(t) for t in self.k_inv]
+        self.lat_caches = [grow(t) for t in self.lat_caches]
         self.free_pages.extend(range(self.num_pages + extra - 1, self.num_pages - 1, -1))
         self.num_pages += extra
         self.max_cache_len = self.num_pages * self.page_size

@@ -58,3 +58,43 @@ class KResidualRMSNorm(BaseInjectedModule):
         from ktransformers_amd._native_seq import rms_combine
         return rms_combine(y, self.weight_f32, self.eps, one_plus=self.one_plus, residual=residual, rows=rows,
                            out_dtype=out_dtype or torch.float32)
+
+
+class KLayerNormBias(BaseInjectedModule):
+    """Layer norm with weight and bias over an fp32 residual stream: (x - mean) / sqrt(var + eps) * w + b, var = the mean of the squared
+    deviations.  Two uses, one operator (include/ktx_hyb.h):
+
+    * in FRONT of a sublayer (`forward(x)`), or as the model's last norm with a row gather (`rows=`): the normed rows in the compute
+      type (`ktx_layer_norm`);
+    * BEHIND a sublayer (`gated_add(x, y, ...)`): x += norm(z), z = the sublayer's result — optionally plus its output bias and plus the
+      weighted rows of a mixture of experts — times sigmoid(gate logits + gate bias) when a gate is given; one launch
+      (`ktx_gated_norm_add`).
+
+    Checkpoint tensors: the module's key (weight) and `<key>.b` (bias, optional)."""
+
+    def __init__(self, key: str, gguf_loader, config, orig_module, prefill_device: str = "cuda", generate_device: str = "cuda",
+                 bias_suffix: str = ".b", **kwargs):
+        BaseInjectedModule.__init__(self, key, gguf_loader, config, orig_module, prefill_device, generate_device, **kwargs)
+        object.__setattr__(self, "eps", float(orig_module.eps))
+        object.__setattr__(self, "bias_suffix", bias_suffix)
+        object.__setattr__(self, "compute_dtype", getattr(config, "compute_dtype", None))
+        object.__setattr__(self, "weight_f32", None)
+        object.__setattr__(self, "bias_f32", None)
+
+    def load(self):
+        import torch
+        dev = torch.device(self.device)
+        object.__setattr__(self, "weight_f32", self.gguf_loader.load_tensor(self.key, device=dev).to(torch.float32).contiguous())
+        if self.gguf_loader.has_tensor(self.key + self.bias_suffix):
+            object.__setattr__(self, "bias_f32",
+                               self.gguf_loader.load_tensor(self.key + self.bias_suffix, device=dev).to(torch.float32).contiguous())
+
+    def forward(self, x, rows=None, out_dtype=None):
+        import torch
+        from ktransformers_amd._native_hyb import layer_norm
+        return layer_norm(x, self.weight_f32, self.bias_f32, self.eps, rows=rows, out_dtype=out_dtype or self.compute_dtype or torch.float32)
+
+    def gated_add(self, x, y=None, ybias=None, gate_logits=None, gate_bias=None, expert_rows=None, pair_pos=None, topk_w=None):
+        from ktransformers_amd._native_hyb import gated_norm_add
+        return gated_norm_add(x, self.weight_f32, self.bias_f32, self.eps, y=y, ybias=ybias, gate_logits=gate_logits, gate_bias=gate_bias,
+                              expert_rows=expert_rows, pair_pos=pair_pos, topk_w=topk_w)

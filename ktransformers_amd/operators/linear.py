@@ -353,3 +353,39 @@ class KLinearDense(BaseInjectedModule):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         from ktransformers_amd._native_seq import dense_gemm
         return dense_gemm(x.reshape(-1, x.shape[-1]), self.w["w"])
+
+
+class KLinearRider(BaseInjectedModule):
+    """A dense linear with bias (`<key>` [out, in], `<key>.b` [out]) whose product can RIDE in another operator's input GEMM: an
+    operator that reads the same input appends `rider.w["w"]` to its own merged weight and hands the rider's columns of the fp32 result
+    back; the bias stays separate (`bias_f32`) so that the consumer's kernel adds it.  `forward(h)` is the stand-alone product
+    (include/ktx_seq.h `ktx_dense_gemm`), bias not added."""
+
+    def __init__(self, key: str, gguf_loader, config, orig_module: nn.Module, prefill_device: str = "cuda", generate_device: str = "cuda",
+                 bias_suffix: str = ".b", **kwargs):
+        BaseInjectedModule.__init__(self, key, gguf_loader, config, orig_module, prefill_device, generate_device, **kwargs)
+        object.__setattr__(self, "compute_dtype", getattr(config, "compute_dtype", torch.bfloat16))
+        object.__setattr__(self, "bias_suffix", bias_suffix)
+        object.__setattr__(self, "bias_f32", None)
+        object.__setattr__(self, "w", {})
+
+    def load(self):
+        dev = torch.device(self.device)
+        self.w["w"] = self.gguf_loader.load_tensor(self.key, device=dev).to(self.compute_dtype).contiguous()
+        if self.gguf_loader.has_tensor(self.key + self.bias_suffix):
+            object.__setattr__(self, "bias_f32",
+                               self.gguf_loader.load_tensor(self.key + self.bias_suffix, device=dev).to(torch.float32).contiguous())
+
+    @property
+    def out_rows(self) -> int:
+        return self.w["w"].shape[0]
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        from ktransformers_amd._native_seq import dense_gemm
+        return dense_gemm(x.reshape(-1, x.shape[-1]), self.w["w"])
+
+
+def merged_input_weight(own: list, rider) -> torch.Tensor:
+    """[own_0 ; own_1 ; ... ; rider.w] as one contiguous [rows, in] weight: all products of one input in one GEMM."""
+    parts = list(own) + ([rider.w["w"]] if rider is not None else [])
+    return torch.cat(parts).contiguous()

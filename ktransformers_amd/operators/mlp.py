@@ -126,3 +126,46 @@ class KDenseMLP(BaseInjectedModule):
         if post_norm is not None and residual is not None:
             return post_norm(y, residual=residual)
         return y
+
+
+class KPolyNormMLP(BaseInjectedModule):
+    """Two-matrix feed-forward with biases and the PolyNorm activation, W_down act(W_up h + b_up) + b_down,
+
+        act(z) = c0 u(z) + c1 u(z^2) + c2 u(z^3) + c3,   u(v) = v / sqrt(mean(v^2) + eps) over the ff entries of a token,
+
+    on an fp32 residual stream (include/ktx_hyb.h `ktx_poly_norm`; the norms are fp32).  A rider's product (operators/linear.py
+    KLinearRider: a linear of the same input) is computed in the up GEMM.  Returns the down product WITHOUT its bias — `down_bias` is
+    for the consumer's kernel to add — and the rider's columns.  Checkpoint tensors: `<key>.up` [ff, width], `<key>.up.b`, `<key>.down`
+    [width, ff], `<key>.down.b`, `<key>.act` [4]."""
+
+    def __init__(self, key: str, gguf_loader, config, orig_module, prefill_device: str = "cuda", generate_device: str = "cuda", **kwargs):
+        BaseInjectedModule.__init__(self, key, gguf_loader, config, orig_module, prefill_device, generate_device, **kwargs)
+        object.__setattr__(self, "eps", float(orig_module.eps))
+        object.__setattr__(self, "compute_dtype", getattr(config, "compute_dtype", torch.bfloat16))
+        object.__setattr__(self, "w", {})
+        object.__setattr__(self, "_merged", {})
+
+    def load(self):
+        ld, dev = self.gguf_loader, torch.device(self.device)
+        for n in ("up", "down"):
+            self.w[n] = ld.load_tensor(f"{self.key}.{n}", device=dev).to(self.compute_dtype).contiguous()
+        for n in ("up.b", "down.b", "act"):
+            self.w[n] = ld.load_tensor(f"{self.key}.{n}", device=dev).to(torch.float32).contiguous() if ld.has_tensor(f"{self.key}.{n}") else None
+        if self.w["act"] is None or self.w["act"].numel() != 4:
+            raise ValueError(f"{self.key}.act: four coefficients expected")
+
+    @property
+    def down_bias(self):
+        return self.w["down.b"]
+
+    def forward(self, h, rider=None):
+        from ktransformers_amd._native_hyb import poly_norm
+        from ktransformers_amd._native_seq import dense_gemm
+        from ktransformers_amd.operators.linear import merged_input_weight
+        k = id(rider) if rider is not None else None
+        if k not in self._merged:
+            self._merged[k] = merged_input_weight([self.w["up"]], rider)
+        F = self.w["up"].shape[0]
+        proj = dense_gemm(h, self._merged[k])
+        a = poly_norm(proj[:, :F], self.w["up.b"], self.w["act"], self.eps, out_dtype=self.compute_dtype)
+        return dense_gemm(a, self.w["down"]), (proj[:, F:] if rider is not None else None)

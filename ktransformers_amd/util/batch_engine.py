@@ -48,7 +48,7 @@ class _DecodeGraph:
         cache, model, dev = engine.cache, engine.model, engine.device
         # the warm-up runs advance the recurrent state of the batch's slots: put it back afterwards (appending the same key rows
         # again changes nothing)
-        keep = [(t, t.clone()) for group in (cache.S, cache.n, cache.m) for t in group if t is not None]
+        keep = [(t, t.clone()) for t in cache.state_tensors()]
         stream = torch.cuda.Stream(device=dev)
         stream.wait_stream(torch.cuda.current_stream(dev))
         with torch.cuda.stream(stream):
