@@ -61,11 +61,16 @@ class CUDAGraphRunner:
         ib = self.input_buffers
         stream = torch.cuda.Stream(device=dev)
         stream.wait_stream(torch.cuda.current_stream(dev))
+        # a cache with recurrent state slots is advanced by every run of the step: the warm-up runs must not count (appending the same
+        # key rows again changes nothing)
+        keep = [(t, t.clone()) for t in past_key_values.state_tensors()] if hasattr(past_key_values, "state_tensors") else []
         with torch.cuda.stream(stream):
             for _ in range(2):   # warm-up outside the capture: lazy handle creation, workspace growth, attribute setting
                 logits = model(ib["cur_token"], ib["position_ids"], past_key_values, ib["cache_position"])
         torch.cuda.current_stream(dev).wait_stream(stream)
         torch.cuda.synchronize(dev)
+        for t, saved in keep:
+            t.copy_(saved)
         self.graph = torch.cuda.CUDAGraph()
         from ktransformers_amd import _native
         _native.TRACE = trace

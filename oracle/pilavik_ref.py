@@ -90,14 +90,15 @@ def latent_attention(P, pre, c, h, eps):
     H, D, R, V, L = c["heads"], c["dim"], c["rot_dim"], c["vdim"], c["kv_rank"]
     pos = torch.arange(T)
     q = (h @ P[pre + "q"].T).view(T, H, D + R)
-    qn, qr = q[..., :D], rotate_pairs(q[..., D:], pos, c["rot"]["base"], c["rot"]["dims"])
+    rot = c.get("rot") or {"base": 1.0, "dims": 0}
+    qn, qr = q[..., :D], rotate_pairs(q[..., D:], pos, rot["base"], rot["dims"])
     dkv = h @ P[pre + "dkv"].T
     lat = unit_rms(dkv[:, :L], eps) * P[pre + "dkv.norm"]
-    kr = rotate_pairs(dkv[:, L:], pos, c["rot"]["base"], c["rot"]["dims"])                    # [T, R]
+    kr = rotate_pairs(dkv[:, L:], pos, rot["base"], rot["dims"])                              # [T, R]
     kn = (lat @ P[pre + "uk"].T).view(T, H, D)
     val = (lat @ P[pre + "uv"].T).view(T, H, V)
     out = torch.zeros(T, H, V, dtype=h.dtype)
-    W = c["mask"]["size"]
+    W = (c.get("mask") or {}).get("size") or T + 1          # no mask: every earlier position is seen
     for i in range(T):
         lo = max(0, i - W + 1)
         for hd in range(H):
@@ -165,8 +166,8 @@ def layer_runs(cfg):
 
 
 def forward(P, cfg, tokens, return_layers=False):
-    """tokens: 1-D LongTensor -> logits [T, vocab] (and the residual stream after every layer run)."""
-    x0 = P["embed"][tokens]
+    """tokens: a list of ids or a 1-D LongTensor -> logits [T, vocab] (and the residual stream after every layer run)."""
+    x0 = P["embed"][torch.as_tensor(tokens, dtype=torch.long)]
     x, trail = x0.clone(), []
     for i, t, first in layer_runs(cfg):
         if first:
@@ -178,3 +179,84 @@ def forward(P, cfg, tokens, return_layers=False):
     eps = cfg["norm"]["eps"]
     logits = layer_norm(x, P["final.norm"], P["final.norm.b"], eps) @ P["head"].T
     return (logits, torch.stack(trail)) if return_layers else logits
+
+
+# ---- small random models for the tests ------------------------------------------------------------------------------------------
+def delta_layer(heads=4, kv_heads=2, dim=16, vdim=16, conv=3, mlp=None):
+    return {"type": "delta", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv}, "mlp": mlp}
+
+
+def attention_layer(heads=3, dim=16, rot_dim=8, vdim=16, kv_rank=24, window=12, rot_dims=None, base=10000.0, scale=None, mlp=None):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank,
+         "scale": scale if scale is not None else (dim + rot_dim) ** -0.5,
+         "rot": {"base": base, "dims": rot_dim if rot_dims is None else rot_dims}}
+    if window:
+        m["mask"] = {"size": window}
+    return {"type": "latent_attention", "mixer": m, "mlp": mlp}
+
+
+def dense_mlp(ff=48):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe_mlp(experts=6, top=2, ff=24, scale=1.5, shared_ff=24):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top, "scale": scale},
+            "shared": {"ff": shared_ff} if shared_ff else None}
+
+
+def make_config(layers, width=32, vocab=61, eps=1e-5, loop=None):
+    return {"architecture": "Pilavik", "width": width, "vocab": vocab, "norm": {"eps": eps}, "layers": layers, "loop": loop}
+
+
+def random_checkpoint(cfg: dict, seed: int = 0) -> dict:
+    """Random bf16-representable weights with the checkpoint's tensor names for a config of the design."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+
+    def mat(o, i, s=None):
+        return (torch.randn(o, i, generator=g) * (s if s is not None else 1.0 / math.sqrt(i))).to(torch.bfloat16)
+
+    def vec(n, mean=0.0, s=0.1):
+        return (mean + torch.randn(n, generator=g) * s).to(torch.bfloat16)
+
+    P = {"embed": mat(cfg["vocab"], W, 1.0), "head": mat(cfg["vocab"], W), "final.norm": vec(W, 1.0), "final.norm.b": vec(W)}
+    if cfg.get("loop"):
+        P["loop.step"] = mat(cfg["loop"]["times"], W, 0.3)
+    for li, layer in enumerate(cfg["layers"]):
+        p, m = f"l{li}.", layer["mixer"]
+        for n in ("norm1", "norm1b") + (("norm2", "norm2b") if layer.get("mlp") else ()):
+            P[p + n], P[p + n + ".b"] = vec(W, 1.0), vec(W)
+        for n in ("rg1",) + (("rg2",) if layer.get("mlp") else ()):
+            P[p + n], P[p + n + ".b"] = mat(W, W), vec(W, 0.5, 0.5)
+        if layer["type"] == "delta":
+            H, G, D, V, K = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
+            P[p + "mix.q"], P[p + "mix.k"], P[p + "mix.v"] = mat(G * D, W, 1.0), mat(G * D, W, 1.0), mat(H * V, W, 1.0)
+            for n, rows in (("q", G * D), ("k", G * D), ("v", H * V)):
+                P[p + f"mix.{n}.conv"] = mat(rows, K, 0.6)
+            P[p + "mix.b"], P[p + "mix.a"], P[p + "mix.g"] = mat(H, W), mat(H, W), mat(H * V, W)
+            P[p + "mix.A_log"], P[p + "mix.dt_bias"] = vec(H, -1.0, 0.7), vec(H, -1.0, 1.0)
+            P[p + "mix.norm"], P[p + "mix.o"] = vec(V, 1.0), mat(W, H * V)
+        else:
+            H, D, R, V, L = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+            P[p + "mix.q"], P[p + "mix.dkv"] = mat(H * (D + R), W, 2.0 / math.sqrt(W)), mat(L + R, W, 2.0 / math.sqrt(W))
+            P[p + "mix.dkv.norm"] = vec(L, 1.0)
+            P[p + "mix.uk"], P[p + "mix.uv"] = mat(H * D, L), mat(H * V, L)
+            P[p + "mix.sink"], P[p + "mix.o"] = vec(H, 0.0, 1.0), mat(W, H * V)
+        c = layer.get("mlp")
+        if c and c["kind"] == "dense":
+            P[p + "mlp.up"], P[p + "mlp.up.b"] = mat(c["ff"], W), vec(c["ff"])
+            P[p + "mlp.down"], P[p + "mlp.down.b"] = mat(W, c["ff"]), vec(W)
+            P[p + "mlp.act"] = torch.tensor([0.6, 0.3, 0.2, 0.1]).to(torch.bfloat16) + vec(4, 0.0, 0.05)
+        elif c:
+            F = c["expert"]["ff"]
+            P[p + "mlp.router"] = mat(c["router"]["experts"], W, 2.0 / math.sqrt(W))
+            for e in range(c["router"]["experts"]):
+                P[p + f"mlp.e{e}.gate"], P[p + f"mlp.e{e}.up"], P[p + f"mlp.e{e}.down"] = mat(F, W), mat(F, W), mat(W, F)
+            if c.get("shared"):
+                SF = c["shared"]["ff"]
+                P[p + "mlp.shared.gate"], P[p + "mlp.shared.up"], P[p + "mlp.shared.down"] = mat(SF, W), mat(SF, W), mat(W, SF)
+    return P
+
+
+def as_double(P: dict) -> dict:
+    return {k: v.double() for k, v in P.items()}
