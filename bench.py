@@ -1696,6 +1696,262 @@ def run_mitotar(args, dev):
     print(json.dumps(line), flush=True)
 
 
+# ---------------------------------------------------------------------------------------------------------------------
+# --pilavik: the hybrid delta-rule / latent-window-attention family with PolyNorm and mixture feed-forwards
+# (models/modeling_pilavik.py) at a few layer sizes, beside Mitotar — the closest existing family: the same fp32 residual, cache
+# manager, step function and graph replay, an attention plus a matrix-memory recurrence per layer — at equal width and depth
+# ---------------------------------------------------------------------------------------------------------------------
+PILAVIK_SIZES = {
+    # per block of 4 layers: delta, delta, attention, delta; feed-forwards dense, moe, moe, moe
+    "w1024": dict(width=1024, d_heads=8, d_kv=4, d_dim=128, d_vdim=128, a_heads=8, a_dim=64, a_rot=32, a_vdim=64, kv_rank=256, window=1024,
+                  ff=2816, experts=16, top=2, e_ff=704, s_ff=704, mitotar="w1024"),
+    "w2048": dict(width=2048, d_heads=16, d_kv=8, d_dim=128, d_vdim=128, a_heads=16, a_dim=128, a_rot=64, a_vdim=128, kv_rank=512,
+                  window=1024, ff=5632, experts=32, top=4, e_ff=704, s_ff=1408, mitotar="w2048"),
+    "w4096": dict(width=4096, d_heads=32, d_kv=8, d_dim=128, d_vdim=128, a_heads=32, a_dim=128, a_rot=64, a_vdim=128, kv_rank=512,
+                  window=2048, ff=11008, experts=64, top=6, e_ff=1024, s_ff=2048, mitotar="w4096"),
+}
+
+
+def pilavik_config(sz, n_layers, vocab=32000):
+    delta = {"type": "delta", "mixer": {"heads": sz["d_heads"], "kv_heads": sz["d_kv"], "dim": sz["d_dim"], "vdim": sz["d_vdim"], "conv": 4}}
+    attn = {"type": "latent_attention",
+            "mixer": {"heads": sz["a_heads"], "dim": sz["a_dim"], "rot_dim": sz["a_rot"], "vdim": sz["a_vdim"], "kv_rank": sz["kv_rank"],
+                      "scale": (sz["a_dim"] + sz["a_rot"]) ** -0.5, "mask": {"size": sz["window"]},
+                      "rot": {"base": 10000.0, "dims": sz["a_rot"]}}}
+    dense = {"kind": "dense", "ff": sz["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": sz["e_ff"]}, "router": {"experts": sz["experts"], "top": sz["top"], "scale": 1.0},
+           "shared": {"ff": sz["s_ff"]}}
+    layers = [dict((delta, delta, attn, delta)[i % 4], mlp=(dense, moe, moe, moe)[i % 4]) for i in range(n_layers)]
+    return {"architecture": "Pilavik", "width": sz["width"], "vocab": vocab, "norm": {"eps": 1e-5}, "layers": layers, "loop": None}
+
+
+class HybRandomLoader:
+    """Random bf16 weights by tensor name for a Pilavik config (names and shapes of models/modeling_pilavik.py's checkpoint)."""
+
+    def __init__(self, cfg, dev):
+        self.dev, self.tensor_device_map, self.shapes = dev, {}, {}
+        W, S = cfg["width"], self.shapes
+        S.update({"embed": (cfg["vocab"], W), "head": (cfg["vocab"], W), "final.norm": (W,), "final.norm.b": (W,)})
+        if cfg.get("loop"):
+            S["loop.step"] = (cfg["loop"]["times"], W)
+        for i, L in enumerate(cfg["layers"]):
+            p, m, c = f"l{i}.", L["mixer"], L.get("mlp")
+            for n in ("norm1", "norm1b") + (("norm2", "norm2b") if c else ()):
+                S[p + n] = S[p + n + ".b"] = (W,)
+            for n in ("rg1",) + (("rg2",) if c else ()):
+                S[p + n], S[p + n + ".b"] = (W, W), (W,)
+            if L["type"] == "delta":
+                H, G, D, V, K = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
+                S.update({p + "mix.q": (G * D, W), p + "mix.k": (G * D, W), p + "mix.v": (H * V, W), p + "mix.g": (H * V, W),
+                          p + "mix.b": (H, W), p + "mix.a": (H, W), p + "mix.q.conv": (G * D, K), p + "mix.k.conv": (G * D, K),
+                          p + "mix.v.conv": (H * V, K), p + "mix.A_log": (H,), p + "mix.dt_bias": (H,), p + "mix.norm": (V,),
+                          p + "mix.o": (W, H * V)})
+            else:
+                H, D, R, V, Lr = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+                S.update({p + "mix.q": (H * (D + R), W), p + "mix.dkv": (Lr + R, W), p + "mix.dkv.norm": (Lr,), p + "mix.uk": (H * D, Lr),
+                          p + "mix.uv": (H * V, Lr), p + "mix.sink": (H,), p + "mix.o": (W, H * V)})
+            if c and c["kind"] == "dense":
+                S.update({p + "mlp.up": (c["ff"], W), p + "mlp.up.b": (c["ff"],), p + "mlp.down": (W, c["ff"]), p + "mlp.down.b": (W,),
+                          p + "mlp.act": (4,)})
+            elif c:
+                F = c["expert"]["ff"]
+                S[p + "mlp.router"] = (c["router"]["experts"], W)
+                for e in range(c["router"]["experts"]):
+                    S.update({p + f"mlp.e{e}.gate": (F, W), p + f"mlp.e{e}.up": (F, W), p + f"mlp.e{e}.down": (W, F)})
+                if c.get("shared"):
+                    SF = c["shared"]["ff"]
+                    S.update({p + "mlp.shared.gate": (SF, W), p + "mlp.shared.up": (SF, W), p + "mlp.shared.down": (W, SF)})
+
+    def has_tensor(self, name):
+        return name in self.shapes
+
+    def load_tensor(self, name, device="cpu"):
+        import zlib
+        shape = self.shapes[name]
+        g = torch.Generator(device=self.dev)
+        g.manual_seed(zlib.crc32(name.encode()))
+        t = torch.randn(shape, generator=g, device=self.dev, dtype=torch.bfloat16)
+        if name.endswith((".dkv.norm", "mix.norm")) or (name.rsplit(".", 1)[-1].startswith("norm") and not name.endswith(".b")):
+            return t.mul_(0.1).add_(1.0)
+        if name.endswith(".act"):
+            return torch.tensor([0.6, 0.3, 0.2, 0.05], device=self.dev, dtype=torch.bfloat16)
+        if name.endswith(("A_log", "dt_bias")):
+            return t.mul_(0.5).sub_(1.0)
+        if name.endswith(".conv"):
+            return t.mul_(0.5)
+        if len(shape) == 1 or name == "embed":
+            return t.mul_(0.1) if name.endswith(".b") else t
+        return t.mul_(shape[-1] ** -0.5)
+
+    def active_params(self, cfg):
+        """Weights one token reads: everything but the embedding table and the experts it does not choose."""
+        n = 0
+        for k, v in self.shapes.items():
+            if k == "embed":
+                continue
+            size = math.prod(v)
+            if ".mlp.e" in k:
+                li = int(k.split(".")[0][1:])
+                r = cfg["layers"][li]["mlp"]["router"]
+                size = size * r["top"] / r["experts"]
+            n += size
+        return n
+
+
+class HybKernelTimer(SeqKernelTimer):
+    """HIP events around every call of the hybrid-decoder and sequence-mixer bindings (see SeqKernelTimer)."""
+    HYB = ("layer_norm", "gated_norm_add", "poly_norm", "silu_mul_rows", "head_gate_norm", "delta_prep", "delta_forward", "latattn_prep",
+           "latattn_forward", "moe_route", "moe_plan", "head_gemm", "expert_gemm", "rows_add")
+    SEQ = ("embed_rows", "dense_gemm")
+
+    def _cost(self, name, a, kw, out):
+        nb = lambda t: t.numel() * t.element_size() if isinstance(t, torch.Tensor) else 0
+        tensors = lambda xs: sum(nb(t) for t in xs)
+        if name == "dense_gemm":
+            M, K = a[0].shape
+            N = a[1].shape[0]
+            return f"dense_gemm M={'prompt' if M > 16 else 'decode'}", 2.0 * M * N * K, M * K * a[0].element_size() + nb(a[1]) + nb(out)
+        if name == "head_gemm":
+            G, N, K = a[2].shape
+            M = a[0].shape[0]
+            return "head_gemm", 2.0 * M * G * N * K, M * G * (K * a[0].element_size() + N * a[3].element_size()) + nb(a[2])
+        if name == "expert_gemm":
+            G, N, K = a[1].shape
+            rows = a[2].pairs
+            touched = min(G, rows)
+            return f"expert_gemm M={'prompt' if rows > 64 else 'decode'}", 2.0 * rows * N * K, rows * K * a[0].element_size() + touched * N * K * a[1].element_size() + nb(out)
+        if name == "latattn_forward":
+            cfg, q, cache = a[0], a[1], a[2]
+            pairs, keys = self.kv_len_of()
+            E = cfg.kv_rank + cfg.rot_dim
+            return name, 2.0 * pairs * cfg.heads * (E + cfg.kv_rank), keys * E * cache.element_size() + nb(q) + nb(out)
+        if name == "delta_forward":
+            cfg, qkv = a[0], a[1]
+            B = a[3].B
+            return name, 6.0 * qkv.shape[0] * cfg.heads * cfg.dim * cfg.vdim, 2.0 * B * cfg.heads * cfg.dim * cfg.vdim * 4 + nb(qkv) + nb(out)
+        outs = out if isinstance(out, (tuple, list)) else (out,)
+        return name, 0.0, tensors(x for x in a if isinstance(x, torch.Tensor)) + tensors(kw.values()) + tensors(outs)
+
+    def __enter__(self):
+        from ktransformers_amd import _native_hyb, _native_seq
+        for mod, names in ((_native_hyb, self.HYB), (_native_seq, self.SEQ)):
+            for name in names:
+                fn = getattr(mod, name)
+                self.saved[(mod, name)] = fn
+
+                def wrapped(*a, _fn=fn, _name=name, **kw):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    out = _fn(*a, **kw)
+                    e1.record()
+                    self.rows.append((e0, e1) + self._cost(_name, a, kw, out))
+                    return out
+                setattr(mod, name, wrapped)
+        return self
+
+    def __exit__(self, *exc):
+        for (mod, name), fn in self.saved.items():
+            setattr(mod, name, fn)
+
+
+def run_pilavik(args, dev):
+    """Prefill (one prompt of --prefill-tokens) and decode (batch 1 and 8 at a 2048-token context) throughput of Pilavik at
+    PILAVIK_SIZES, each beside Mitotar of equal width and depth, with a per-kernel table and the fraction of its roofline (bf16 MFMA
+    peak or HBM peak, whichever bounds).  Random weights, synthetic tokens.  Prints one JSON line; the whole record goes to
+    bench_pilavik.json beside this file."""
+    import contextlib
+    import io
+    from ktransformers_amd.models import load_model
+    from ktransformers_amd.util.batch_engine import BatchEngine
+
+    n_layers, T, ctx = args.layers or 4, args.prefill_tokens, 2048
+    sizes = [s for s in (args.pilavik.split(",") if args.pilavik != "all" else PILAVIK_SIZES) if s in PILAVIK_SIZES]
+    record = {"metric": "pilavik_prefill_decode", "unit": "tok/s", "layers": n_layers, "prefill_tokens": T, "decode_ctx": ctx,
+              "dtype": "bf16 weights / activations / latent cache, fp32 residual, scores, router, state", "data": "synthetic", "sizes": {}}
+
+    def timed_ms(fn, reps):
+        fn()
+        torch.cuda.synchronize(dev)
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize(dev)
+            ts.append((time.perf_counter() - t0) * 1e3)
+        return sorted(ts)[len(ts) // 2]
+
+    def measure(cfg, loader, timer_cls, window):
+        with contextlib.redirect_stdout(io.StringIO()):
+            model, config, entry = load_model(cfg, dtype=torch.bfloat16, device=str(dev), loader=loader)
+        cache = entry.make_cache(config, 8 * (ctx + 64) + T, 16, torch.bfloat16, str(dev))
+        eng = BatchEngine(model, cache, use_graph=not args.no_graph)
+        g = torch.Generator().manual_seed(5)
+        prompt = torch.randint(0, 32000, (T,), generator=g).tolist()
+        state = {"pairs": 0, "keys": 0}
+        seen = lambda n: min(n, window) if window else n
+
+        def prefill():
+            state.update(pairs=sum(seen(i + 1) for i in range(T)), keys=T)
+            eng.step([{"id": "p", "tokens": prompt, "want": [T - 1]}], ["p"])
+        ms = timed_ms(prefill, 3)
+        with timer_cls(lambda: (state["pairs"], state["keys"])) as kt:
+            prefill()
+        res = {"prefill": {"tok_s": round(T / ms * 1e3, 1), "ms": round(ms, 3), "per_kernel": kt.table(ms)}}
+        for B in (1, 8):
+            ids = [f"d{b}" for b in range(B)]
+            ctx_prompt = torch.randint(0, 32000, (ctx,), generator=g).tolist()
+            eng.step([{"id": r, "tokens": ctx_prompt, "want": []} for r in ids])
+
+            def decode():
+                n = seen(cache.seq_len(ids[0]))
+                state.update(pairs=B * n, keys=B * n)
+                eng.step([{"id": r, "tokens": [7], "want": [0]} for r in ids])
+            ms = timed_ms(decode, 20)
+            eng.use_graph = False           # the per-kernel pass brackets eager launches
+            with timer_cls(lambda: (state["pairs"], state["keys"])) as kt:
+                decode()
+            eng.use_graph = not args.no_graph
+            res[f"decode_bs{B}"] = {"tok_s": round(B / ms * 1e3, 1), "ms_per_step": round(ms, 3), "per_kernel": kt.table(ms),
+                                    "graph": eng.use_graph}
+            for r in ids:
+                cache.release(r)
+        del model, cache, eng
+        torch.cuda.empty_cache()
+        return res
+
+    for name in sizes:
+        sz = PILAVIK_SIZES[name]
+        cfg = pilavik_config(sz, n_layers)
+        loader = HybRandomLoader(cfg, dev)
+        res = measure(cfg, loader, HybKernelTimer, sz["window"])
+        active = loader.active_params(cfg)
+        res["weights_GB"] = round(sum(math.prod(v) for k, v in loader.shapes.items() if k != "embed") * 2 / 1e9, 3)
+        res["active_weights_GB"] = round(active * 2 / 1e9, 3)
+        res["decode_bs1"]["frac_of_hbm_peak"] = round(active * 2 / (res["decode_bs1"]["ms_per_step"] * 1e-3) / (HBM_PEAK_GBS * 1e9), 4)
+        try:
+            ms_ = MITOTAR_SIZES[sz["mitotar"]]
+            layer = {"type": "parallel", "mlp": {"kind": "dense", "ff": ms_["ff"]},
+                     "mixer": {"left": {"heads": ms_["heads"], "kv_heads": ms_["kv_heads"], "dim": ms_["dim"], "vdim": ms_["dim"],
+                                        "scale": ms_["dim"] ** -0.5, "q_temp": {"coef": 0.4, "every": 128}},
+                               "right": {"heads": ms_["r_heads"], "dim": ms_["r_dim"], "vdim": ms_["r_vdim"], "gate_cap": 15.0}}}
+            mcfg = {"architecture": "Mitotar", "width": ms_["width"], "vocab": 32000, "norm": {"eps": 1e-5}, "layers": [layer] * n_layers}
+            res["mitotar"] = measure(mcfg, SeqRandomLoader(mcfg, dev), SeqKernelTimer, 0)
+        except Exception as e:      # the comparison must not lose the new family's numbers
+            res["mitotar"] = {"error": f"{type(e).__name__}: {e}"}
+        record["sizes"][name] = res
+        log(f"[pilavik] {name}: prefill {res['prefill']['tok_s']} tok/s, decode bs1 {res['decode_bs1']['tok_s']} tok/s, "
+            f"bs8 {res['decode_bs8']['tok_s']} tok/s")
+    with open(os.path.join(ROOT, "bench_pilavik.json"), "w") as f:
+        json.dump(record, f, indent=1)
+    line = {"metric": record["metric"], "unit": "tok/s", "layers": n_layers, "data": "synthetic",
+            "sizes": {k: {"prefill": v["prefill"]["tok_s"], "decode_bs1": v["decode_bs1"]["tok_s"], "decode_bs8": v["decode_bs8"]["tok_s"],
+                          "mitotar_prefill": v["mitotar"].get("prefill", {}).get("tok_s"),
+                          "mitotar_decode_bs1": v["mitotar"].get("decode_bs1", {}).get("tok_s"),
+                          "mitotar_decode_bs8": v["mitotar"].get("decode_bs8", {}).get("tok_s")}
+                      for k, v in record["sizes"].items()}}
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -1735,6 +1991,10 @@ def main():
                     help="instead of the default workload: prefill / decode throughput of the Mitotar family (sigmoid head-mixing attention "
                          "+ mLSTM mixers) at layer sizes from MITOTAR_SIZES (comma-separated, or 'all'), beside a dense DeepSeek of equal "
                          "size; one JSON line, detail in bench_mitotar.json")
+    ap.add_argument("--pilavik", default="", metavar="SIZES",
+                    help="instead of the default workload: prefill / decode throughput of the Pilavik family (gated delta rule + latent "
+                         "window attention, PolyNorm and mixture feed-forwards) at layer sizes from PILAVIK_SIZES (comma-separated, or "
+                         "'all'), beside Mitotar of equal width and depth; one JSON line, detail in bench_pilavik.json")
     ap.add_argument("--pmc-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--trace-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
@@ -1756,6 +2016,10 @@ def main():
     if args.mitotar:
         torch.cuda.set_device(dev)
         run_mitotar(args, dev)
+        return
+    if args.pilavik:
+        torch.cuda.set_device(dev)
+        run_pilavik(args, dev)
         return
     torch.cuda.set_device(dev)
     if args.pmc_child:

@@ -97,6 +97,16 @@ int ktx_latattn_forward(const ktx_latattn_config* cfg, int T, const float* d_q, 
                         const int32_t* d_pos, const int32_t* d_page_indptr, const int32_t* d_page_indices, const float* d_sink,
                         int nsplit, float* d_scratch, void* d_out, int out_dtype, ktx_stream_t stream);
 
+/* The same operator on the matrix cores, for prompts, portions and decode steps: request b's query rows q_indptr[b] .. q_indptr[b+1]
+ * (at most max_q_len tokens; T in all) start at position pos0[b].  The (token, head) pairs of a request are the rows of one query
+ * matrix against the shared latent rows; workgroups of 64 rows walk 32-key tiles: bf16 MFMA for q . row and for weights x rows (q
+ * rounded to bf16), scores / mask / softmax in fp32.  nsplit key ranges per workgroup row (scratch as above), then merged with the sink.
+ * Eligible: bf16 cache, kv_rank 64 / 128 / 256 / 512, rot_dim a multiple of 8 up to 128; ktx_latattn_forward serves everything else. */
+int ktx_latattn_mfma_eligible(const ktx_latattn_config* cfg);
+int ktx_latattn_mfma(const ktx_latattn_config* cfg, int B, int T, int max_q_len, const float* d_q, const void* d_cache,
+                     const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_page_indptr, const int32_t* d_page_indices,
+                     const float* d_sink, int nsplit, float* d_scratch, void* d_out, int out_dtype, ktx_stream_t stream);
+
 /* ---- mixture of experts ---------------------------------------------------------------------------------------------------- */
 /* s = sigmoid(logits[t]) (fp32 rows of stride ldl, E experts); the `top` largest (lowest index first on ties) ->
  * topk_idx int32 [T][top], topk_w fp32 [T][top] = s / (sum of the chosen s + sum_eps) * scale. */

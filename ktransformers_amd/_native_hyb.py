@@ -35,6 +35,8 @@ lib.ktx_delta_prep.argtypes = [C.POINTER(_DeltaConfig), _I, _I, _P, _P, _P, _P, 
 lib.ktx_delta_forward.argtypes = [C.POINTER(_DeltaConfig), _I, _P, _P, _P, _P, _P, _P, _P, _P]
 lib.ktx_latattn_prep.argtypes = [C.POINTER(_LatAttnConfig), _I, _P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P]
 lib.ktx_latattn_forward.argtypes = [C.POINTER(_LatAttnConfig), _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _P]
+lib.ktx_latattn_mfma_eligible.argtypes = [C.POINTER(_LatAttnConfig)]
+lib.ktx_latattn_mfma.argtypes = [C.POINTER(_LatAttnConfig), _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _P]
 lib.ktx_moe_route.argtypes = [_I, _I, _I, _F, _F, _P, _L, _P, _P, _P]
 lib.ktx_moe_plan.argtypes = [_I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P]
 lib.ktx_grouped_gemm.argtypes = [_I, _I, _I, _I, _P, _I, _L, _L, _P, _P, _I, _P, _I, _L, _L, _P, _P, _P, _P, _I, _P]
@@ -205,6 +207,23 @@ def latattn_forward(cfg: _LatAttnConfig, q: torch.Tensor, cache: torch.Tensor, b
     check(lib.ktx_latattn_forward(C.byref(cfg), T, q.data_ptr(), cache.data_ptr(), batch.tok_req.data_ptr(), batch.positions.data_ptr(),
                                   batch.page_indptr.data_ptr(), batch.page_indices.data_ptr(), sink.data_ptr(), int(nsplit), _ptr(scratch),
                                   out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(q.device)))
+    return out
+
+
+def latattn_mfma_eligible(cfg: _LatAttnConfig) -> bool:
+    return bool(lib.ktx_latattn_mfma_eligible(C.byref(cfg)))
+
+
+def latattn_mfma(cfg: _LatAttnConfig, q: torch.Tensor, cache: torch.Tensor, batch, sink: torch.Tensor, nsplit: int = 1,
+                 out_dtype=torch.bfloat16) -> torch.Tensor:
+    """The matrix-core kernel, prompts and decode steps (ktx_latattn_mfma) -> [T, heads * kv_rank] of out_dtype."""
+    _f32(q, "latattn_mfma q"), _f32(sink, "latattn_mfma sink")
+    T, L = q.shape[0], cfg.kv_rank
+    out = torch.empty((T, cfg.heads * L), dtype=out_dtype, device=q.device)
+    scratch = torch.empty((nsplit, T, cfg.heads, L + 2), dtype=torch.float32, device=q.device) if nsplit > 1 else None
+    check(lib.ktx_latattn_mfma(C.byref(cfg), batch.B, T, int(batch.max_q_len), q.data_ptr(), cache.data_ptr(), batch.q_indptr.data_ptr(),
+                               batch.pos0.data_ptr(), batch.page_indptr.data_ptr(), batch.page_indices.data_ptr(), sink.data_ptr(),
+                               int(nsplit), _ptr(scratch), out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(q.device)))
     return out
 
 

@@ -234,17 +234,32 @@ __global__ void __launch_bounds__(256) delta_fwd_kernel(ktx_delta_config c, cons
     const int d = wave * DPW + r;
     S[r] = (carried && d < D && col < V) ? Sp[(size_t)d * V + col] : 0.f;
   }
-  auto stage = [&](int t, int par) {
+  // the next token's inputs travel global -> registers (fetch, issued a whole token ahead so that the memory latency is off the
+  // sequential path) -> LDS (commit, into the buffer the token after the current one reads)
+  constexpr int NKQ = (2 * DP + 255) / 256;
+  float pre_kq[NKQ], pre_misc = 0.f;
+  auto fetch = [&](int t) {
     const float* row = qkv + (size_t)t * C;
-    for (int e = tid; e < 2 * DP; e += 256) {
-      const int which = e / DP, d = e % DP;          // 0: k, 1: q
-      kq[par][e] = d < D ? row[(which ? 0 : GD) + kh * D + d] : 0.f;
+#pragma unroll
+    for (int i = 0; i < NKQ; i++) {
+      const int e = tid + i * 256, which = e / DP, d = e % DP;          // 0: k, 1: q
+      pre_kq[i] = (e < 2 * DP && d < D) ? row[(which ? 0 : GD) + kh * D + d] : 0.f;
     }
-    if (tid < 64) vv[par][tid] = (vs * 64 + tid) < V ? row[2 * GD + h * V + vs * 64 + tid] : 0.f;
-    if (tid == 64) vv[par][64] = gb[(size_t)t * 2 * H + h];
-    if (tid == 65) vv[par][65] = gb[(size_t)t * 2 * H + H + h];
+    if (tid < 64) pre_misc = (vs * 64 + tid) < V ? row[2 * GD + h * V + vs * 64 + tid] : 0.f;
+    else if (tid == 64) pre_misc = gb[(size_t)t * 2 * H + h];
+    else if (tid == 65) pre_misc = gb[(size_t)t * 2 * H + H + h];
   };
-  stage(t0, 0);
+  auto commit = [&](int par) {
+#pragma unroll
+    for (int i = 0; i < NKQ; i++) {
+      const int e = tid + i * 256;
+      if (e < 2 * DP) kq[par][e] = pre_kq[i];
+    }
+    if (tid < 66) vv[par][tid] = pre_misc;
+  };
+  fetch(t0);
+  commit(0);
+  if (t0 + 1 < t1) fetch(t0 + 1);
   __syncthreads();
   for (int t = t0; t < t1; t++) {
     const int par = (t - t0) & 1;
@@ -263,7 +278,8 @@ __global__ void __launch_bounds__(256) delta_fwd_kernel(ktx_delta_config c, cons
     red[par][wave][0][lane] = pk;
     red[par][wave][1][lane] = pq;
     if (lane == 0) redkq[par][wave] = dkq;
-    if (t + 1 < t1) stage(t + 1, par ^ 1);
+    if (t + 1 < t1) commit(par ^ 1);
+    if (t + 2 < t1) fetch(t + 2);
     __syncthreads();
     const float kS = (red[par][0][0][lane] + red[par][1][0][lane]) + (red[par][2][0][lane] + red[par][3][0][lane]);
     const float qS = (red[par][0][1][lane] + red[par][1][1][lane]) + (red[par][2][1][lane] + red[par][3][1][lane]);
@@ -453,6 +469,169 @@ __global__ void __launch_bounds__(256) latattn_merge_kernel(int T, int H, int L,
     }
     st_elem(out, ((size_t)t * H + h) * L + l, a / den);
   }
+}
+
+
+// The same attention on the matrix cores (bf16 latent cache).  The latent rows are keys AND values of every head, so the (token, head)
+// pairs of a request are the rows of one long query matrix against shared keys: a workgroup takes 64 consecutive rows (its four
+// wavefronts one 16-row MFMA tile each, query fragments resident in registers) and walks 32-key tiles of the union of its rows'
+// windows: the tile is staged once in LDS row-major (scores) and transposed (values); scores, mask, running maximum and sum in fp32
+// (DPP reductions inside the 16-lane column groups), weights through a per-wavefront LDS tile into the second product.  Key ranges
+// (blockIdx.z) leave unnormalised partial sums that latattn_merge_kernel joins with the sink.
+constexpr int LM_KT = 32, LM_PST = LM_KT + 8;
+template <int NT, typename OT>
+__global__ void __launch_bounds__(256) latattn_mfma_kernel(ktx_latattn_config c, int T, int row_tiles, const float* __restrict__ q,
+                                                           const bf16_t* __restrict__ cache, const int32_t* __restrict__ q_indptr,
+                                                           const int32_t* __restrict__ pos0, const int32_t* __restrict__ page_indptr,
+                                                           const int32_t* __restrict__ page_indices, const float* __restrict__ sink,
+                                                           int nsplit, float* __restrict__ scratch, OT* __restrict__ out) {
+  constexpr int L = NT * 16, KSMAX = NT / 2 + 4;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lm_raw[];
+  const int H = c.heads, E = L + c.rot_dim, EP = (E + 31) & ~31, EPP = EP + 8, KS = EP / 32;
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(lm_raw);            // [LM_KT][EPP]
+  bf16_t* Vt = Ks + (size_t)LM_KT * EPP;                      // [L][LM_PST]
+  bf16_t* Ps = Vt + (size_t)L * LM_PST;                       // [4][16][LM_PST]
+  int* rowidx = reinterpret_cast<int*>(Ps + 4 * 16 * LM_PST); // [LM_KT]
+  const int b = blockIdx.x / row_tiles, rt = blockIdx.x % row_tiles, z = blockIdx.z;
+  const int t0 = q_indptr[b], rows_total = (q_indptr[b + 1] - t0) * H, r0 = rt * 64;
+  if (r0 >= rows_total) return;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
+  const int p0 = pos0[b];
+  const int tok_lo = r0 / H, tok_hi = (min(rows_total, r0 + 64) - 1) / H;
+  const int klo = c.window > 0 ? max(0, p0 + tok_lo - c.window + 1) : 0, khi = p0 + tok_hi + 1;
+  const int per = (((khi - klo + nsplit - 1) / nsplit) + LM_KT - 1) / LM_KT * LM_KT;
+  const int j0 = klo + z * per, j1 = min(khi, j0 + per);
+  const int rw0 = r0 + wave * 16;
+  const bool active = rw0 < rows_total;
+  // query fragments: lane = (row l16, 8 consecutive entries lq * 8 ..) of every 32-entry step
+  sq_v8bf qf[KSMAX];
+  {
+    const int ar = rw0 + l16;
+    const float* qrow = q + ((size_t)t0 * H + ar) * E;
+#pragma unroll
+    for (int kk = 0; kk < KSMAX; kk++) {
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const int e = kk * 32 + lq * 8 + i;
+        v[i] = (kk < KS && ar < rows_total && e < E) ? qrow[e] : 0.f;
+      }
+      union { uint4 u; sq_v8bf f; } cv;
+      cv.u.x = ktx_pk_bf16(v[0], v[1]); cv.u.y = ktx_pk_bf16(v[2], v[3]); cv.u.z = ktx_pk_bf16(v[4], v[5]); cv.u.w = ktx_pk_bf16(v[6], v[7]);
+      qf[kk] = cv.f;
+    }
+  }
+  // the four rows this lane holds of the score / output tiles (C layout: row lq * 4 + r, column l16)
+  int prow[4], lorow[4], hrow[4];
+  bool vrow[4];
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    const int cr = rw0 + lq * 4 + r;
+    vrow[r] = cr < rows_total;
+    prow[r] = p0 + cr / H;
+    hrow[r] = cr % H;
+    lorow[r] = c.window > 0 ? max(0, prow[r] - c.window + 1) : 0;
+  }
+  float mrun[4], lrun[4];
+  v4f acc[NT];
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    mrun[r] = -INFINITY;
+    lrun[r] = 0.f;
+  }
+#pragma unroll
+  for (int n = 0; n < NT; n++) acc[n] = (v4f){0.f, 0.f, 0.f, 0.f};
+  const int32_t* pages = page_indices + page_indptr[b];
+  const int segs = EP / 8;
+  bf16_t* Pw = Ps + (size_t)wave * 16 * LM_PST;
+  for (int jt = j0; jt < j1; jt += LM_KT) {
+    const int nk = min(LM_KT, j1 - jt);
+    __syncthreads();
+    if (tid < LM_KT) {
+      const int j = jt + tid;
+      rowidx[tid] = tid < nk ? pages[j / c.page_size] * c.page_size + j % c.page_size : -1;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < LM_KT * segs; idx += 256) {
+      const int key = idx / segs, e0 = (idx % segs) * 8;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      const int row = rowidx[key];
+      if (row >= 0 && e0 < E) v = *reinterpret_cast<const uint4*>(cache + (size_t)row * E + e0);
+      *reinterpret_cast<uint4*>(Ks + (size_t)key * EPP + e0) = v;
+      if (e0 < L) {
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) Vt[(size_t)(e0 + i) * LM_PST + key] = (bf16_t)((w[i >> 1] >> ((i & 1) * 16)) & 0xffffu);
+      }
+    }
+    __syncthreads();
+    if (active) {
+      v4f s0 = (v4f){0.f, 0.f, 0.f, 0.f}, s1 = s0;
+#pragma unroll
+      for (int kk = 0; kk < KSMAX; kk++) {
+        if (kk < KS) {
+          const sq_v8bf b0 = *reinterpret_cast<const sq_v8bf*>(Ks + (size_t)l16 * EPP + kk * 32 + lq * 8);
+          const sq_v8bf b1 = *reinterpret_cast<const sq_v8bf*>(Ks + (size_t)(16 + l16) * EPP + kk * 32 + lq * 8);
+          s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[kk], b0, s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[kk], b1, s1, 0, 0, 0);
+        }
+      }
+      const int ja = jt + l16, jb = ja + 16;
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const bool oka = vrow[r] && ja < j1 && ja >= lorow[r] && ja <= prow[r];
+        const bool okb = vrow[r] && jb < j1 && jb >= lorow[r] && jb <= prow[r];
+        const float sa = oka ? s0[r] * c.scale : -INFINITY, sb = okb ? s1[r] * c.scale : -INFINITY;
+        const float mt = row16_max(fmaxf(sa, sb));
+        const float mn = fmaxf(mrun[r], mt);
+        const float base = mn == -INFINITY ? 0.f : mn;
+        const float wa = oka ? __expf(sa - base) : 0.f, wb = okb ? __expf(sb - base) : 0.f;
+        const float cr = mrun[r] == -INFINITY ? 0.f : __expf(mrun[r] - base);
+        lrun[r] = lrun[r] * cr + row16_sum(wa + wb);
+        mrun[r] = mn;
+#pragma unroll
+        for (int n = 0; n < NT; n++) acc[n][r] *= cr;
+        Pw[(lq * 4 + r) * LM_PST + l16] = to_bf16_rne(wa);
+        Pw[(lq * 4 + r) * LM_PST + 16 + l16] = to_bf16_rne(wb);
+      }
+    }
+    __syncthreads();
+    if (active) {
+      const sq_v8bf pf = *reinterpret_cast<const sq_v8bf*>(Pw + (size_t)l16 * LM_PST + lq * 8);
+#pragma unroll
+      for (int n = 0; n < NT; n++) {
+        const sq_v8bf vb = *reinterpret_cast<const sq_v8bf*>(Vt + (size_t)(n * 16 + l16) * LM_PST + lq * 8);
+        acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vb, acc[n], 0, 0, 0);
+      }
+    }
+  }
+  if (!active) return;
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    if (!vrow[r]) continue;
+    const int cr = rw0 + lq * 4 + r;
+    const size_t grow = (size_t)t0 * H + cr;             // (token, head) row of q / out
+    if (nsplit == 1) {
+      const float sk = sink[hrow[r]], M = fmaxf(mrun[r], sk);
+      const float f = mrun[r] == -INFINITY ? 0.f : expf(mrun[r] - M);
+      const float inv = f / (lrun[r] * f + expf(sk - M));
+#pragma unroll
+      for (int n = 0; n < NT; n++) st_elem(out, grow * L + n * 16 + l16, acc[n][r] * inv);
+    } else {
+      float* part = scratch + ((size_t)z * T * H + grow) * (L + 2);
+#pragma unroll
+      for (int n = 0; n < NT; n++) part[n * 16 + l16] = acc[n][r];
+      if (l16 == 0) {
+        part[L] = mrun[r];
+        part[L + 1] = lrun[r];
+      }
+    }
+  }
+}
+
+size_t latattn_mfma_lds(const ktx_latattn_config& c) {
+  const int E = c.kv_rank + c.rot_dim, EP = (E + 31) & ~31;
+  return ((size_t)LM_KT * (EP + 8) + (size_t)c.kv_rank * LM_PST + 4 * 16 * LM_PST) * 2 + LM_KT * 4;
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -843,6 +1022,56 @@ int ktx_latattn_forward(const ktx_latattn_config* cfg, int T, const float* d_q, 
     else KTX_LA_GO(bf16_t, bf16_t);
   }
 #undef KTX_LA_GO
+  KTX_HIP(hipGetLastError());
+  if (nsplit > 1) {
+    const dim3 mg(T, cfg->heads);
+    if (out_dtype == KTX_SEQ_F32) latattn_merge_kernel<float><<<mg, 256, 0, st>>>(T, cfg->heads, L, nsplit, d_scratch, d_sink, (float*)d_out);
+    else latattn_merge_kernel<bf16_t><<<mg, 256, 0, st>>>(T, cfg->heads, L, nsplit, d_scratch, d_sink, (bf16_t*)d_out);
+    KTX_HIP(hipGetLastError());
+  }
+  return 0;
+}
+
+int ktx_latattn_mfma_eligible(const ktx_latattn_config* c) {
+  if (!c || c->cache_dtype != KTX_SEQ_BF16) return 0;
+  const int L = c->kv_rank, E = L + c->rot_dim;
+  if (!(L == 64 || L == 128 || L == 256 || L == 512) || E % 8 != 0) return 0;
+  if (((E + 31) / 32) > (L / 16) / 2 + 4) return 0;
+  return latattn_mfma_lds(*c) <= 150 * 1024;
+}
+
+int ktx_latattn_mfma(const ktx_latattn_config* cfg, int B, int T, int max_q_len, const float* d_q, const void* d_cache,
+                     const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_page_indptr, const int32_t* d_page_indices,
+                     const float* d_sink, int nsplit, float* d_scratch, void* d_out, int out_dtype, ktx_stream_t stream) {
+  if (latattn_check(cfg, "ktx_latattn_mfma")) return -1;
+  KTX_REQUIRE(ktx_latattn_mfma_eligible(cfg), "ktx_latattn_mfma: bf16 cache, kv_rank 64 / 128 / 256 / 512, rot_dim a multiple of 8 up to 128");
+  KTX_REQUIRE(B >= 0 && T >= 0 && max_q_len >= 0 && d_q && d_cache && d_q_indptr && d_pos0 && d_page_indptr && d_page_indices && d_sink &&
+                  d_out && dtype_ok(out_dtype),
+              "ktx_latattn_mfma: null pointer");
+  KTX_REQUIRE(nsplit >= 1 && nsplit <= 65535 && (nsplit == 1 || d_scratch), "ktx_latattn_mfma: nsplit >= 1, scratch when > 1");
+  if (B == 0 || T == 0 || max_q_len == 0) return 0;
+  const int row_tiles = (int)(((int64_t)max_q_len * cfg->heads + 63) / 64);
+  const dim3 grid((unsigned)B * row_tiles, 1, nsplit);
+  const size_t lds = latattn_mfma_lds(*cfg);
+  hipStream_t st = (hipStream_t)stream;
+  const int L = cfg->kv_rank;
+#define KTX_LM_GO(NT, OT)                                                                                                       \
+  do {                                                                                                                          \
+    KTX_HIP(ktx_set_max_lds((const void*)latattn_mfma_kernel<NT, OT>, 150 * 1024));                                             \
+    latattn_mfma_kernel<NT, OT><<<grid, 256, lds, st>>>(*cfg, T, row_tiles, d_q, (const bf16_t*)d_cache, d_q_indptr, d_pos0,    \
+                                                        d_page_indptr, d_page_indices, d_sink, nsplit, d_scratch, (OT*)d_out);  \
+  } while (0)
+#define KTX_LM_NT(OT)             \
+  do {                            \
+    if (L == 64) KTX_LM_GO(4, OT);  \
+    else if (L == 128) KTX_LM_GO(8, OT); \
+    else if (L == 256) KTX_LM_GO(16, OT); \
+    else KTX_LM_GO(32, OT);       \
+  } while (0)
+  if (out_dtype == KTX_SEQ_F32) KTX_LM_NT(float);
+  else KTX_LM_NT(bf16_t);
+#undef KTX_LM_NT
+#undef KTX_LM_GO
   KTX_HIP(hipGetLastError());
   if (nsplit > 1) {
     const dim3 mg(T, cfg->heads);

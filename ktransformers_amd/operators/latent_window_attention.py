@@ -23,7 +23,9 @@ from ktransformers_amd.operators.linear import merged_input_weight
 
 class KLatentWindowAttention(BaseInjectedModule):
     TARGET_WORKGROUPS = 1024
-    KEYS_PER_SPLIT = 256
+    KEYS_PER_SPLIT = 64
+    MFMA_KEYS_PER_SPLIT = 64
+    USE_MATRIX_CORES = True
 
     def __init__(self, key: str, gguf_loader, config, orig_module: nn.Module, prefill_device: str = "cuda", generate_device: str = "cuda",
                  **kwargs):
@@ -71,7 +73,7 @@ class KLatentWindowAttention(BaseInjectedModule):
     def forward(self, h: torch.Tensor, batch, cache, cache_idx: int, rider=None):
         """h [T, width] in the compute type.  Returns (W_o(attention) fp32 [T, width], the rider's product or None); the step's latent
         rows are appended to the cache."""
-        from ktransformers_amd._native_hyb import head_gemm, latattn_forward, latattn_prep
+        from ktransformers_amd._native_hyb import head_gemm, latattn_forward, latattn_mfma, latattn_mfma_eligible, latattn_prep
         from ktransformers_amd._native_seq import dense_gemm
         H, D, R, V, L = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank
         cfg, T = self._config(cache), h.shape[0]
@@ -82,8 +84,14 @@ class KLatentWindowAttention(BaseInjectedModule):
         latattn_prep(cfg, proj, 0, c_off, self.w["lat_norm"], self.w["inv_freq"], batch.positions, batch.cache_loc, lat, q)
         head_gemm(proj, D + R, self.w["ukT"], q, L + R)          # q_lat[h] = W_uk[h]^T q_unrotated[h]
         span = batch.max_kv_len if not self.window else min(batch.max_kv_len, self.window)
-        nsplit = max(1, min(self.TARGET_WORKGROUPS // max(T, 1), (span + self.KEYS_PER_SPLIT - 1) // self.KEYS_PER_SPLIT))
-        o_lat = latattn_forward(cfg, q, lat, batch, self.w["sink"], nsplit=nsplit, out_dtype=self.compute_dtype)
+        if self.USE_MATRIX_CORES and lat.dtype == torch.bfloat16 and latattn_mfma_eligible(cfg):
+            # workgroups of 64 (token, head) rows x key ranges, enough of them to fill the chip
+            blocks = batch.B * ((batch.max_q_len * H + 63) // 64)
+            nsplit = max(1, min(self.TARGET_WORKGROUPS // max(blocks, 1), (span + self.MFMA_KEYS_PER_SPLIT - 1) // self.MFMA_KEYS_PER_SPLIT))
+            o_lat = latattn_mfma(cfg, q, lat, batch, self.w["sink"], nsplit=nsplit, out_dtype=self.compute_dtype)
+        else:
+            nsplit = max(1, min(self.TARGET_WORKGROUPS // max(T, 1), (span + self.KEYS_PER_SPLIT - 1) // self.KEYS_PER_SPLIT))
+            o_lat = latattn_forward(cfg, q, lat, batch, self.w["sink"], nsplit=nsplit, out_dtype=self.compute_dtype)
         o = torch.empty((T, H * V), dtype=self.compute_dtype, device=h.device)
         head_gemm(o_lat, L, self.w["uv"], o, V)
         return dense_gemm(o, self.w["o"]), (proj[:, c_off + L + R:] if rider is not None else None)

@@ -234,8 +234,10 @@ def test_delta_rule_remembers_far_tokens():
         assert rel(_mixer_in_portions(op, cache, x, F32, [250, 100] + [1] * 50), r) < 2e-5
 
 
+# the bf16 runs of the kv_rank 64 / 128 / 256 rows take the matrix-core kernel, everything else the vector-ALU one
 ATTN_SIZES = [(3, 16, 8, 16, 24, 12, None), (5, 12, 6, 10, 9, 5, 4), (1, 8, 4, 8, 8, 1, 0), (4, 32, 16, 32, 64, None, None),
-              (2, 16, 8, 24, 40, 70, None), (6, 64, 32, 64, 64, 33, None)]
+              (2, 16, 8, 24, 40, 70, None), (6, 64, 32, 64, 64, 33, None), (5, 16, 8, 16, 128, 20, 6), (16, 8, 24, 8, 256, 47, None),
+              (1, 16, 16, 16, 64, 3, None), (20, 8, 8, 8, 64, None, None)]
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
@@ -250,21 +252,34 @@ def test_latent_attention_whole_portions_and_window(dtype, H, D, Rd, V, L, windo
     tol = 2e-5 if dtype == F32 else 3e-2
     for sizes in ([T], [1] * T, [2] * 45, [7, 1, 30, 2, 50], [89, 1]):
         assert rel(_mixer_in_portions(op, cache, h, dtype, sizes), ref) < tol, sizes
-    op.KEYS_PER_SPLIT = 4               # several workgroups share a token's keys and are merged
+    op.KEYS_PER_SPLIT = op.MFMA_KEYS_PER_SPLIT = 4               # several workgroups share a token's keys and are merged
     try:
         assert rel(_mixer_in_portions(op, cache, h, dtype, [60] + [1] * 30), ref) < tol
+        assert rel(_mixer_in_portions(op, cache, h, dtype, [33, 57]), ref) < tol
     finally:
-        del op.KEYS_PER_SPLIT
+        del op.KEYS_PER_SPLIT, op.MFMA_KEYS_PER_SPLIT
+    if dtype == BF16:                   # both kernels, the same cache rows: they differ by the rounding of the weights alone
+        from ktransformers_amd._native_hyb import latattn_mfma_eligible
+        took_matrix_cores = latattn_mfma_eligible(op._config(cache))
+        assert took_matrix_cores == (L in (64, 128, 256, 512))
+        a = _mixer_in_portions(op, cache, h, dtype, [50, 40])
+        op.USE_MATRIX_CORES = False
+        try:
+            b = _mixer_in_portions(op, cache, h, dtype, [50, 40])
+        finally:
+            del op.USE_MATRIX_CORES
+        assert rel(a, b) < (1.5e-2 if took_matrix_cores else 1e-7)
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("L", [8, 64])
 @pytest.mark.parametrize("window,query,back", [(16, 40, 15), (16, 40, 16), (16, 15, 15), (16, 16, 16), (8, 8, 7), (8, 8, 8), (33, 64, 32),
-                                               (33, 64, 33), (5, 4, 4), (1, 9, 0), (1, 9, 1)])
-def test_one_key_at_the_window_edge_stands_out(dtype, window, query, back):
+                                               (33, 64, 33), (5, 4, 4), (1, 9, 0), (1, 9, 1), (40, 100, 39), (40, 100, 40)])
+def test_one_key_at_the_window_edge_stands_out(dtype, window, query, back, L):
     """The rotated key part is not normed: a token whose input is scaled up gets a score far above all others, so the query `back`
     positions after it takes its value alone when it is inside the window (back < window) and must not see it when it is one place
     outside.  Page size 8: the key sits at, before and after page borders.  As a prompt, and with the query decoded alone."""
-    cfg = R.make_config([R.attention_layer(heads=2, dim=8, rot_dim=8, vdim=8, kv_rank=8, window=window, rot_dims=0, scale=1.0)], width=24)
+    cfg = R.make_config([R.attention_layer(heads=2, dim=8, rot_dim=8, vdim=8, kv_rank=L, window=window, rot_dims=0, scale=1.0)], width=24)
     P = R.random_checkpoint(cfg, 9)
     P["l0.mix.sink"] = torch.full((2,), -30.0).to(BF16)
     op, cache, Pd = _operator(cfg, 9, dtype, P=P)
@@ -275,7 +290,7 @@ def test_one_key_at_the_window_edge_stands_out(dtype, window, query, back):
     c = cfg["layers"][0]["mixer"]
     # sign of the boosted key's rotated score for the query (rot_dims = 0: no dependence on the positions)
     qr = (h[query].double() @ Pd["l0.mix.q"].T).view(2, 16)[:, 8:]
-    kr = h[key].double() @ Pd["l0.mix.dkv"].T[:, 8:]
+    kr = h[key].double() @ Pd["l0.mix.dkv"].T[:, L:]
     if back > 0:
         h[key] = h[key] * (60.0 if float((qr @ kr).sum()) > 0 else -60.0)
     ref = R.latent_attention(Pd, "l0.mix.", c, h.double(), 1e-5)
