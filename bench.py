@@ -1801,7 +1801,7 @@ class HybRandomLoader:
 class HybKernelTimer(SeqKernelTimer):
     """HIP events around every call of the hybrid-decoder and sequence-mixer bindings (see SeqKernelTimer)."""
     HYB = ("layer_norm", "gated_norm_add", "poly_norm", "silu_mul_rows", "head_gate_norm", "delta_prep", "delta_forward", "latattn_prep",
-           "latattn_forward", "moe_route", "moe_plan", "head_gemm", "expert_gemm", "rows_add")
+           "latattn_forward", "latattn_mfma", "moe_route", "moe_plan", "head_gemm", "expert_gemm", "rows_add")
     SEQ = ("embed_rows", "dense_gemm")
 
     def _cost(self, name, a, kw, out):
@@ -1820,7 +1820,7 @@ class HybKernelTimer(SeqKernelTimer):
             rows = a[2].pairs
             touched = min(G, rows)
             return f"expert_gemm M={'prompt' if rows > 64 else 'decode'}", 2.0 * rows * N * K, rows * K * a[0].element_size() + touched * N * K * a[1].element_size() + nb(out)
-        if name == "latattn_forward":
+        if name in ("latattn_forward", "latattn_mfma"):
             cfg, q, cache = a[0], a[1], a[2]
             pairs, keys = self.kv_len_of()
             E = cfg.kv_rank + cfg.rot_dim

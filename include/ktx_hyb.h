@@ -58,7 +58,8 @@ typedef struct ktx_delta_config {
 /* Per token, between the input projection and the recurrence: the convolution over time (channels = q | k | v, C = 2 kv_heads dim +
  * heads vdim; taps fp32 [C][taps], last column = the current token; inputs before a request's first NEW token come from its slot of
  * conv_state fp32 [slots][taps - 1][C] when pos0 > 0 and are zero otherwise), silu, the unit vectors -> qkv fp32 [T][C]; and per head
- * decay g = exp(-exp(A_log) softplus(a + dt_bias)) and step beta = sigmoid(b) -> gb fp32 [T][2 heads] (g | beta).
+ * decay g = exp(-exp(A_log) softplus(a + dt_bias)) and step beta = sigmoid(b), per key head k . q -> gb fp32 [T][2 heads + kv_heads]
+ * (g | beta | k . q).
  * proj: fp32 rows of stride ldp with q, k, v, b, a at their offsets.  Then ktx_delta_conv_update moves the state on (second launch). */
 int ktx_delta_prep(const ktx_delta_config* cfg, int B, int T, const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_slot,
                    const int32_t* d_tok_req, const float* d_proj, int64_t ldp, int q_off, int k_off, int v_off, int b_off, int a_off,
@@ -67,6 +68,7 @@ int ktx_delta_prep(const ktx_delta_config* cfg, int B, int T, const int32_t* d_q
 
 /* Per head, token by token from the slot's state S fp32 [slots][heads][dim][vdim] (zero when pos0 == 0, whatever the slot holds):
  *   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q       (q, k of head h / (heads / kv_heads))
+ * (evaluated as o = (g S)^T q + u (k . q): both read-outs of the decayed state are taken before the write).
  * o fp32 [T][heads * vdim].  dim <= 256. */
 int ktx_delta_forward(const ktx_delta_config* cfg, int B, const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_slot,
                       const float* d_qkv, const float* d_gb, float* d_S, float* d_o, ktx_stream_t stream);
@@ -114,10 +116,12 @@ int ktx_moe_route(int T, int E, int top, float scale, float sum_eps, const float
                   float* d_topk_w, ktx_stream_t stream);
 
 /* Sort the T * top (token, choice) pairs by expert: group_off int32 [E + 1]; sorted_tok int32 [pairs] = the token of each sorted row;
- * pair_pos int32 [pairs] = the sorted row of pair t * top + k; tiles of tile_m rows that never span two experts:
+ * pair_pos int32 [pairs] = the sorted row of pair t * top + k; sorted_group int32 [pairs] = the expert of each sorted row; tiles of
+ * tile_m rows that never span two experts:
  * tile_group / tile_row0 int32 [pairs / tile_m + E + 1], their number in num_tiles[0].  One workgroup; E <= 4096. */
 int ktx_moe_plan(int T, int E, int top, int tile_m, const int32_t* d_topk_idx, int32_t* d_group_off, int32_t* d_sorted_tok,
-                 int32_t* d_pair_pos, int32_t* d_tile_group, int32_t* d_tile_row0, int32_t* d_num_tiles, ktx_stream_t stream);
+                 int32_t* d_pair_pos, int32_t* d_sorted_group, int32_t* d_tile_group, int32_t* d_tile_row0, int32_t* d_num_tiles,
+                 ktx_stream_t stream);
 
 enum { KTX_GG_TILE_M = 64 };
 
@@ -131,6 +135,12 @@ int ktx_grouped_gemm(int G, int M, int N, int K, const void* d_A, int a_dtype, i
                      const void* d_W, int w_dtype, void* d_Y, int y_dtype, int64_t ldy, int64_t y_goff, const int32_t* d_group_off,
                      const int32_t* d_tile_group, const int32_t* d_tile_row0, const int32_t* d_num_tiles, int max_tiles,
                      ktx_stream_t stream);
+
+/* The ragged products for a handful of rows (decode steps), streaming each row's weights once: Y[r] = W_g A[a_rows ? a_rows[r] : r]
+ * with g = row_group[r].  glu != 0: W_g is [2N][K] (gate rows, then up rows) and Y[r][n] = silu(gate_n . a) * (up_n . a) — the
+ * activation of a GLU expert in the same launch.  fp32 accumulation on the vector ALUs; any N, K. */
+int ktx_grouped_gemv(int R, int N, int K, const void* d_A, int a_dtype, int64_t lda, const int32_t* d_a_rows, const void* d_W, int w_dtype,
+                     void* d_Y, int y_dtype, int64_t ldy, const int32_t* d_row_group, int glu, ktx_stream_t stream);
 
 #ifdef __cplusplus
 }

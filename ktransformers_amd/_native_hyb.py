@@ -38,7 +38,8 @@ lib.ktx_latattn_forward.argtypes = [C.POINTER(_LatAttnConfig), _I, _P, _P, _P, _
 lib.ktx_latattn_mfma_eligible.argtypes = [C.POINTER(_LatAttnConfig)]
 lib.ktx_latattn_mfma.argtypes = [C.POINTER(_LatAttnConfig), _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _P]
 lib.ktx_moe_route.argtypes = [_I, _I, _I, _F, _F, _P, _L, _P, _P, _P]
-lib.ktx_moe_plan.argtypes = [_I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P]
+lib.ktx_moe_plan.argtypes = [_I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P]
+lib.ktx_grouped_gemv.argtypes = [_I, _I, _I, _P, _I, _L, _P, _P, _I, _P, _I, _L, _P, _I, _P]
 lib.ktx_grouped_gemm.argtypes = [_I, _I, _I, _I, _P, _I, _L, _L, _P, _P, _I, _P, _I, _L, _L, _P, _P, _P, _P, _I, _P]
 
 TILE_M = 64
@@ -150,7 +151,7 @@ def delta_config(heads: int, kv_heads: int, dim: int, vdim: int, taps: int, unit
 
 def delta_prep(cfg: _DeltaConfig, proj: torch.Tensor, offs: dict, taps: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor,
                batch, conv_state: torch.Tensor | None):
-    """-> (qkv fp32 [T, C], gb fp32 [T, 2 heads]); the slots' convolution state moves on (ktx_delta_prep)."""
+    """-> (qkv fp32 [T, C], gb fp32 [T, 2 heads + kv_heads]); the slots' convolution state moves on (ktx_delta_prep)."""
     pp, ldp = _rows_f32(proj, "delta_prep proj")
     _f32(taps, "taps"), _f32(A_log, "A_log"), _f32(dt_bias, "dt_bias"), _f32(conv_state, "conv_state")
     T = proj.shape[0]
@@ -160,7 +161,7 @@ def delta_prep(cfg: _DeltaConfig, proj: torch.Tensor, offs: dict, taps: torch.Te
     if conv_state is not None and tuple(conv_state.shape[1:]) != (max(cfg.taps - 1, 1), Cn):
         raise KtxError("delta_prep: conv_state must be [slots, taps - 1, C]")
     qkv = torch.empty((T, Cn), dtype=torch.float32, device=proj.device)
-    gb = torch.empty((T, 2 * cfg.heads), dtype=torch.float32, device=proj.device)
+    gb = torch.empty((T, 2 * cfg.heads + cfg.kv_heads), dtype=torch.float32, device=proj.device)
     check(lib.ktx_delta_prep(C.byref(cfg), batch.B, T, batch.q_indptr.data_ptr(), batch.pos0.data_ptr(), batch.slot.data_ptr(),
                              batch.tok_req.data_ptr(), pp, ldp, offs["q"], offs["k"], offs["v"], offs["b"], offs["a"], taps.data_ptr(),
                              A_log.data_ptr(), dt_bias.data_ptr(), _ptr(conv_state), qkv.data_ptr(), gb.data_ptr(), _stream_ptr(proj.device)))
@@ -238,7 +239,7 @@ def moe_route(logits: torch.Tensor, top: int, scale: float, sum_eps: float):
 
 
 class MoePlan:
-    __slots__ = ("group_off", "sorted_tok", "pair_pos", "tile_group", "tile_row0", "num_tiles", "max_tiles", "pairs")
+    __slots__ = ("group_off", "sorted_tok", "pair_pos", "sorted_group", "tile_group", "tile_row0", "num_tiles", "max_tiles", "pairs")
 
 
 def moe_plan(topk_idx: torch.Tensor, E: int) -> MoePlan:
@@ -247,14 +248,14 @@ def moe_plan(topk_idx: torch.Tensor, E: int) -> MoePlan:
     p = MoePlan()
     p.pairs = T * top
     p.max_tiles = p.pairs // TILE_M + min(E, p.pairs) + 1
-    meta = torch.empty(E + 1 + 2 * p.pairs + 2 * p.max_tiles + 1, dtype=torch.int32, device=topk_idx.device)
+    meta = torch.empty(E + 1 + 3 * p.pairs + 2 * p.max_tiles + 1, dtype=torch.int32, device=topk_idx.device)
     at = 0
-    for name, n in (("group_off", E + 1), ("sorted_tok", p.pairs), ("pair_pos", p.pairs), ("tile_group", p.max_tiles),
+    for name, n in (("group_off", E + 1), ("sorted_tok", p.pairs), ("pair_pos", p.pairs), ("sorted_group", p.pairs), ("tile_group", p.max_tiles),
                     ("tile_row0", p.max_tiles), ("num_tiles", 1)):
         setattr(p, name, meta[at:at + n])
         at += n
     check(lib.ktx_moe_plan(T, E, top, TILE_M, topk_idx.data_ptr(), p.group_off.data_ptr(), p.sorted_tok.data_ptr(), p.pair_pos.data_ptr(),
-                           p.tile_group.data_ptr(), p.tile_row0.data_ptr(), p.num_tiles.data_ptr(), _stream_ptr(topk_idx.device)))
+                           p.sorted_group.data_ptr(), p.tile_group.data_ptr(), p.tile_row0.data_ptr(), p.num_tiles.data_ptr(), _stream_ptr(topk_idx.device)))
     return p
 
 
@@ -276,10 +277,23 @@ def head_gemm(a: torch.Tensor, a_goff: int, w: torch.Tensor, out: torch.Tensor, 
     return out
 
 
-def expert_gemm(a: torch.Tensor, w: torch.Tensor, plan: MoePlan, gather: bool, out_dtype=torch.float32) -> torch.Tensor:
-    """Sorted row r (expert g = the group it falls in) : out[r] = a[plan.sorted_tok[r] if gather else r] @ w[g]^T.  w [E, N, K]."""
+GEMV_MAX_ROWS = 64      # up to this many (token, choice) pairs a step's expert products stream the weights per row instead of tiling
+
+
+def expert_gemm(a: torch.Tensor, w: torch.Tensor, plan: MoePlan, gather: bool, out_dtype=torch.float32, glu: bool = False) -> torch.Tensor:
+    """Sorted row r (expert g = the group it falls in) : out[r] = a[plan.sorted_tok[r] if gather else r] @ w[g]^T.  w [E, N, K].
+    glu (only for steps of at most GEMV_MAX_ROWS pairs): w[g] = [gate ; up] and out[r] = silu(gate a) * (up a), [pairs, N / 2]."""
     G, N, K = w.shape
     _gg_types(a, w, out_dtype)
+    if plan.pairs <= GEMV_MAX_ROWS:
+        n_out = N // 2 if glu else N
+        out = torch.empty((plan.pairs, n_out), dtype=out_dtype, device=a.device)
+        check(lib.ktx_grouped_gemv(plan.pairs, n_out, K, a.data_ptr(), SEQ_DTYPE[a.dtype], a.stride(0),
+                                   plan.sorted_tok.data_ptr() if gather else None, w.data_ptr(), SEQ_DTYPE[w.dtype], out.data_ptr(),
+                                   SEQ_DTYPE[out_dtype], out.stride(0), plan.sorted_group.data_ptr(), int(glu), _stream_ptr(a.device)))
+        return out
+    if glu:
+        raise KtxError("expert_gemm: the fused activation is the streaming form's (at most GEMV_MAX_ROWS pairs)")
     out = torch.empty((plan.pairs, N), dtype=out_dtype, device=a.device)
     check(lib.ktx_grouped_gemm(G, plan.pairs, N, K, a.data_ptr(), SEQ_DTYPE[a.dtype], a.stride(0), 0,
                                plan.sorted_tok.data_ptr() if gather else None, w.data_ptr(), SEQ_DTYPE[w.dtype], out.data_ptr(),

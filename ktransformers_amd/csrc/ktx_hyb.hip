@@ -175,10 +175,17 @@ __global__ void __launch_bounds__(256) delta_prep_kernel(ktx_delta_config c, con
   }
   __syncthreads();
   for (int e = tid; e < C; e += 256) qkv[(size_t)t * C + e] = ch[e];
+  float* gbt = gb + (size_t)t * (2 * c.heads + c.kv_heads);
   for (int h = tid; h < c.heads; h += 256) {
     const float a = proj[(size_t)t * ldp + a_off + h] + dt_bias[h];
-    gb[(size_t)t * 2 * c.heads + h] = expf(-expf(A_log[h]) * softplus_f32(a));
-    gb[(size_t)t * 2 * c.heads + c.heads + h] = sigmoid_f32(proj[(size_t)t * ldp + b_off + h]);
+    gbt[h] = expf(-expf(A_log[h]) * softplus_f32(a));
+    gbt[c.heads + h] = sigmoid_f32(proj[(size_t)t * ldp + b_off + h]);
+  }
+  for (int j = wave; j < c.kv_heads; j += 4) {      // k . q per key head: the recurrence's read-out of the token's own write
+    float s = 0.f;
+    for (int d = lane; d < c.dim; d += 64) s += ch[(size_t)j * c.dim + d] * ch[GD + (size_t)j * c.dim + d];
+    s = wave_sum(s);
+    if (lane == 0) gbt[2 * c.heads + j] = s;
   }
 }
 
@@ -215,14 +222,13 @@ __global__ void __launch_bounds__(256) delta_fwd_kernel(ktx_delta_config c, cons
                                                         float* __restrict__ Sg, float* __restrict__ o) {
   constexpr int DP = 4 * DPW;
   __shared__ float kq[2][2 * DP];          // k | q of the token's key head
-  __shared__ float vv[2][64 + 2];          // the value slice, then g and beta
+  __shared__ float vv[2][64 + 3];          // the value slice, then g, beta and k . q
   __shared__ float red[2][4][2][64];
-  __shared__ float redkq[2][4];
   const int VS = (c.vdim + 63) / 64;
   const int vs = blockIdx.x % VS, h = (blockIdx.x / VS) % c.heads, b = blockIdx.x / (VS * c.heads);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int D = c.dim, V = c.vdim, H = c.heads, GD = c.kv_heads * D, C = 2 * GD + H * V;
-  const int kh = h / (H / c.kv_heads);
+  const int kh = h / (H / c.kv_heads), NGB = 2 * H + c.kv_heads;
   const int col = vs * 64 + lane;
   const int t0 = q_indptr[b], t1 = q_indptr[b + 1];
   if (t1 <= t0) return;
@@ -246,8 +252,9 @@ __global__ void __launch_bounds__(256) delta_fwd_kernel(ktx_delta_config c, cons
       pre_kq[i] = (e < 2 * DP && d < D) ? row[(which ? 0 : GD) + kh * D + d] : 0.f;
     }
     if (tid < 64) pre_misc = (vs * 64 + tid) < V ? row[2 * GD + h * V + vs * 64 + tid] : 0.f;
-    else if (tid == 64) pre_misc = gb[(size_t)t * 2 * H + h];
-    else if (tid == 65) pre_misc = gb[(size_t)t * 2 * H + H + h];
+    else if (tid == 64) pre_misc = gb[(size_t)t * NGB + h];
+    else if (tid == 65) pre_misc = gb[(size_t)t * NGB + H + h];
+    else if (tid == 66) pre_misc = gb[(size_t)t * NGB + 2 * H + kh];
   };
   auto commit = [&](int par) {
 #pragma unroll
@@ -255,7 +262,7 @@ __global__ void __launch_bounds__(256) delta_fwd_kernel(ktx_delta_config c, cons
       const int e = tid + i * 256;
       if (e < 2 * DP) kq[par][e] = pre_kq[i];
     }
-    if (tid < 66) vv[par][tid] = pre_misc;
+    if (tid < 67) vv[par][tid] = pre_misc;
   };
   fetch(t0);
   commit(0);
@@ -263,31 +270,28 @@ __global__ void __launch_bounds__(256) delta_fwd_kernel(ktx_delta_config c, cons
   __syncthreads();
   for (int t = t0; t < t1; t++) {
     const int par = (t - t0) & 1;
-    const float g = vv[par][64], beta = vv[par][65], val = vv[par][lane];
+    const float g = vv[par][64], beta = vv[par][65], kdq = vv[par][66], val = vv[par][lane];
     float kr[DPW];
-    float pk = 0.f, pq = 0.f, dkq = 0.f;
+    float pk = 0.f, pq = 0.f;
 #pragma unroll
     for (int r = 0; r < DPW; r++) {
       const float kd = kq[par][wave * DPW + r], qd = kq[par][DP + wave * DPW + r];
       kr[r] = kd;
       S[r] *= g;
-      pk += kd * S[r];
-      pq += qd * S[r];
-      dkq += kd * qd;
+      pk = fmaf(kd, S[r], pk);
+      pq = fmaf(qd, S[r], pq);
     }
     red[par][wave][0][lane] = pk;
     red[par][wave][1][lane] = pq;
-    if (lane == 0) redkq[par][wave] = dkq;
     if (t + 1 < t1) commit(par ^ 1);
     if (t + 2 < t1) fetch(t + 2);
     __syncthreads();
     const float kS = (red[par][0][0][lane] + red[par][1][0][lane]) + (red[par][2][0][lane] + red[par][3][0][lane]);
     const float qS = (red[par][0][1][lane] + red[par][1][1][lane]) + (red[par][2][1][lane] + red[par][3][1][lane]);
-    const float kdq = (redkq[par][0] + redkq[par][1]) + (redkq[par][2] + redkq[par][3]);
     const float u = beta * (val - kS);
 #pragma unroll
-    for (int r = 0; r < DPW; r++) S[r] += kr[r] * u;
-    if (wave == 0 && col < V) o[((size_t)t * H + h) * V + col] = qS + u * kdq;
+    for (int r = 0; r < DPW; r++) S[r] = fmaf(kr[r], u, S[r]);
+    if (wave == 0 && col < V) o[((size_t)t * H + h) * V + col] = fmaf(u, kdq, qS);
   }
 #pragma unroll
   for (int r = 0; r < DPW; r++) {
@@ -692,8 +696,9 @@ __global__ void __launch_bounds__(256) moe_route_kernel(int T, int E, int top, f
 // one workgroup sorts the pairs by expert (counting sort in LDS) and lays the row tiles out
 __global__ void __launch_bounds__(1024) moe_plan_kernel(int pairs, int E, int top, int tile_m, const int32_t* __restrict__ idx,
                                                         int32_t* __restrict__ group_off, int32_t* __restrict__ sorted_tok,
-                                                        int32_t* __restrict__ pair_pos, int32_t* __restrict__ tile_group,
-                                                        int32_t* __restrict__ tile_row0, int32_t* __restrict__ num_tiles) {
+                                                        int32_t* __restrict__ pair_pos, int32_t* __restrict__ sorted_group,
+                                                        int32_t* __restrict__ tile_group, int32_t* __restrict__ tile_row0,
+                                                        int32_t* __restrict__ num_tiles) {
   extern __shared__ int32_t pl[];          // counts [E] | offsets [E + 1] | cursor [E]
   int32_t* cnt = pl;
   int32_t* off = pl + E;
@@ -723,6 +728,7 @@ __global__ void __launch_bounds__(1024) moe_plan_kernel(int pairs, int E, int to
     const int e = idx[i];
     const int p = off[e] + atomicAdd(&cur[e], 1);
     sorted_tok[p] = i / top;
+    sorted_group[p] = e;
     pair_pos[i] = p;
   }
 }
@@ -836,6 +842,72 @@ __global__ void __launch_bounds__(256) grouped_gemm_kernel(int M, int N, int K, 
         const int m = m0 + wm + i * 16 + lq * 4 + r, n = n0 + wn + j * 16 + l16;
         if (m < m_end && n < N) st_elem(Y, (size_t)m * ldy + n, acc[i][j][r]);
       }
+}
+
+// the same products for a handful of rows (decode steps): no tile, the weights stream once per row.  Workgroup = (8 output columns,
+// one sorted row); a wavefront owns two columns and its lanes stride over K in 16-byte pieces.  glu: column f pairs rows f and
+// F + f of the group's [2F][K] matrix and writes silu(first) * second.
+template <typename AT, typename CT, typename YT>
+__global__ void __launch_bounds__(256) grouped_gemv_kernel(int N, int K, const AT* __restrict__ A, int64_t lda,
+                                                           const int32_t* __restrict__ a_rows, const CT* __restrict__ W, int w_rows,
+                                                           YT* __restrict__ Y, int64_t ldy, const int32_t* __restrict__ row_group,
+                                                           int glu, bool vec) {
+  const int r = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const AT* a = A + (size_t)(a_rows ? a_rows[r] : r) * lda;
+  const CT* Wg = W + (size_t)row_group[r] * w_rows * K;
+#pragma unroll
+  for (int c2 = 0; c2 < 2; c2++) {
+    const int n = blockIdx.x * 8 + wave * 2 + c2;
+    if (n >= N) continue;
+    const CT* w0 = Wg + (size_t)n * K;
+    const CT* w1 = Wg + (size_t)(N + n) * K;
+    float s0 = 0.f, s1 = 0.f;
+    if (vec) {
+      for (int k = lane * 8; k < K; k += 512) {
+        float av[8], wv[8], uv[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) av[i] = ld_elem(a, k + i);
+        if constexpr (sizeof(CT) == 2) {
+          const uint4 p = *reinterpret_cast<const uint4*>(w0 + k);
+          const uint32_t pw[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            wv[2 * i] = ktx_lo_f32(pw[i]);
+            wv[2 * i + 1] = ktx_hi_f32(pw[i]);
+          }
+          if (glu) {
+            const uint4 p1 = *reinterpret_cast<const uint4*>(w1 + k);
+            const uint32_t pu[4] = {p1.x, p1.y, p1.z, p1.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+              uv[2 * i] = ktx_lo_f32(pu[i]);
+              uv[2 * i + 1] = ktx_hi_f32(pu[i]);
+            }
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; i++) {
+            wv[i] = w0[k + i];
+            if (glu) uv[i] = w1[k + i];
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          s0 = fmaf(av[i], wv[i], s0);
+          if (glu) s1 = fmaf(av[i], uv[i], s1);
+        }
+      }
+    } else {
+      for (int k = lane; k < K; k += 64) {
+        const float av = ld_elem(a, k);
+        s0 = fmaf(av, ld_elem(w0, k), s0);
+        if (glu) s1 = fmaf(av, ld_elem(w1, k), s1);
+      }
+    }
+    s0 = wave_sum(s0);
+    if (glu) s1 = wave_sum(s1);
+    if (lane == 0) st_elem(Y, (size_t)r * ldy + n, glu ? silu_f32(s0) * s1 : s0);
+  }
 }
 
 int dtype_ok(int d) { return d == KTX_SEQ_F32 || d == KTX_SEQ_BF16; }
@@ -1093,12 +1165,14 @@ int ktx_moe_route(int T, int E, int top, float scale, float sum_eps, const float
 }
 
 int ktx_moe_plan(int T, int E, int top, int tile_m, const int32_t* d_topk_idx, int32_t* d_group_off, int32_t* d_sorted_tok,
-                 int32_t* d_pair_pos, int32_t* d_tile_group, int32_t* d_tile_row0, int32_t* d_num_tiles, ktx_stream_t stream) {
+                 int32_t* d_pair_pos, int32_t* d_sorted_group, int32_t* d_tile_group, int32_t* d_tile_row0, int32_t* d_num_tiles,
+                 ktx_stream_t stream) {
   KTX_REQUIRE(T >= 0 && E > 0 && E <= 4096 && top > 0 && tile_m > 0 && d_topk_idx && d_group_off && d_sorted_tok && d_pair_pos &&
-                  d_tile_group && d_tile_row0 && d_num_tiles,
+                  d_sorted_group && d_tile_group && d_tile_row0 && d_num_tiles,
               "ktx_moe_plan: arguments");
   moe_plan_kernel<<<1, 1024, (size_t)(3 * E + 1) * 4, (hipStream_t)stream>>>(T * top, E, top, tile_m, d_topk_idx, d_group_off, d_sorted_tok,
-                                                                              d_pair_pos, d_tile_group, d_tile_row0, d_num_tiles);
+                                                                              d_pair_pos, d_sorted_group, d_tile_group, d_tile_row0,
+                                                                              d_num_tiles);
   KTX_HIP(hipGetLastError());
   return 0;
 }
@@ -1134,6 +1208,34 @@ int ktx_grouped_gemm(int G, int M, int N, int K, const void* d_A, int a_dtype, i
     KTX_GG_GO(float, float, float);
   }
 #undef KTX_GG_GO
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_grouped_gemv(int R, int N, int K, const void* d_A, int a_dtype, int64_t lda, const int32_t* d_a_rows, const void* d_W, int w_dtype,
+                     void* d_Y, int y_dtype, int64_t ldy, const int32_t* d_row_group, int glu, ktx_stream_t stream) {
+  KTX_REQUIRE(R >= 0 && N > 0 && K > 0 && d_A && d_W && d_Y && d_row_group, "ktx_grouped_gemv: N, K > 0, pointers");
+  KTX_REQUIRE(dtype_ok(a_dtype) && dtype_ok(w_dtype) && dtype_ok(y_dtype), "ktx_grouped_gemv: unknown element type");
+  KTX_REQUIRE(R <= 65535, "ktx_grouped_gemv: up to 65535 rows");
+  if (R == 0) return 0;
+  const size_t asz = a_dtype == KTX_SEQ_F32 ? 4 : 2, wsz = w_dtype == KTX_SEQ_F32 ? 4 : 2;
+  const bool vec = aligned16(d_W) && ((size_t)K * wsz) % 16 == 0 && K % 8 == 0 && aligned16(d_A) && (lda * asz) % 16 == 0;
+  const dim3 grid((N + 7) / 8, R);
+  const int w_rows = glu ? 2 * N : N;
+  hipStream_t st = (hipStream_t)stream;
+#define KTX_GV_GO(AT, CT, YT)                                                                                                          \
+  grouped_gemv_kernel<AT, CT, YT><<<grid, 256, 0, st>>>(N, K, (const AT*)d_A, lda, d_a_rows, (const CT*)d_W, w_rows, (YT*)d_Y, ldy, \
+                                                        d_row_group, glu, vec)
+  if (w_dtype == KTX_SEQ_BF16) {
+    if (a_dtype == KTX_SEQ_F32 && y_dtype == KTX_SEQ_F32) KTX_GV_GO(float, bf16_t, float);
+    else if (a_dtype == KTX_SEQ_F32) KTX_GV_GO(float, bf16_t, bf16_t);
+    else if (y_dtype == KTX_SEQ_F32) KTX_GV_GO(bf16_t, bf16_t, float);
+    else KTX_GV_GO(bf16_t, bf16_t, bf16_t);
+  } else {
+    KTX_REQUIRE(a_dtype == KTX_SEQ_F32 && y_dtype == KTX_SEQ_F32, "ktx_grouped_gemv: an fp32 product takes and writes fp32");
+    KTX_GV_GO(float, float, float);
+  }
+#undef KTX_GV_GO
   KTX_HIP(hipGetLastError());
   return 0;
 }

@@ -52,7 +52,7 @@ class KSigmoidRoutedMoE(BaseInjectedModule):
     def forward(self, h: torch.Tensor, rider=None):
         """h [T, width] in the compute type -> (shared expert's output fp32 [T, width] or None, the rider's product or None,
         expert_rows fp32 [T * top, width] in sorted order, pair_pos int32 [T * top], topk_w fp32 [T, top])."""
-        from ktransformers_amd._native_hyb import expert_gemm, moe_plan, moe_route, silu_mul_rows
+        from ktransformers_amd._native_hyb import GEMV_MAX_ROWS, expert_gemm, moe_plan, moe_route, silu_mul_rows
         from ktransformers_amd._native_seq import dense_gemm
         k = id(rider) if rider is not None else None
         if k not in self._merged:
@@ -62,8 +62,10 @@ class KSigmoidRoutedMoE(BaseInjectedModule):
         proj = dense_gemm(h, self._merged[k])
         idx, wts = moe_route(proj[:, :E], self.top, self.route_scale, self.sum_eps)
         plan = moe_plan(idx, E)
-        gu = expert_gemm(h, self.w["gate_up"], plan, gather=True)
-        act = silu_mul_rows(gu, out_dtype=self.compute_dtype)
+        if plan.pairs <= GEMV_MAX_ROWS:      # decode steps: the weights stream once per pair, the activation in the same launch
+            act = expert_gemm(h, self.w["gate_up"], plan, gather=True, out_dtype=self.compute_dtype, glu=True)
+        else:
+            act = silu_mul_rows(expert_gemm(h, self.w["gate_up"], plan, gather=True), out_dtype=self.compute_dtype)
         rows = expert_gemm(act, self.w["down"], plan, gather=False)
         shared = None
         if SF:
