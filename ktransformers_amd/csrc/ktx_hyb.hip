@@ -17,6 +17,9 @@ namespace {
 #include "ktx_seq_dev.inc"
 
 __device__ __forceinline__ float silu_f32(float z) { return z / (1.0f + expf(-z)); }
+// A workgroup barrier that orders LDS traffic only: the wavefront's own LDS operations have completed, global loads it has in flight
+// (a prefetch for a later step) stay in flight — __syncthreads() would wait for them too.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 __device__ __forceinline__ float softplus_f32(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
@@ -212,18 +215,19 @@ __global__ void __launch_bounds__(256) delta_conv_update_kernel(ktx_delta_config
   }
 }
 
-// the recurrence: workgroup = (request, head, 64 value columns); wavefront = a quarter of the dim rows, lane = value column; the state
+// the recurrence: workgroup = (request, head, 64 value columns); wavefront = dim / NW rows (NW = 4 or 8), lane = value column; the state
 // slice stays in registers; ONE barrier per token: both read-outs (S^T k and S^T q of the decayed state) are taken before the write,
-// o = (g S)^T q + u (k . q).
-template <int DPW>
-__global__ void __launch_bounds__(256) delta_fwd_kernel(ktx_delta_config c, const int32_t* __restrict__ q_indptr,
+// o = (g S)^T q + u (k . q).  The tokens' inputs are staged through LDS a chunk ahead.
+template <int DPW, int NW>
+__global__ void __launch_bounds__(NW * 64) delta_fwd_kernel(ktx_delta_config c, const int32_t* __restrict__ q_indptr,
                                                         const int32_t* __restrict__ pos0, const int32_t* __restrict__ slot,
                                                         const float* __restrict__ qkv, const float* __restrict__ gb,
                                                         float* __restrict__ Sg, float* __restrict__ o) {
-  constexpr int DP = 4 * DPW;
-  __shared__ float kq[2][2 * DP];          // k | q of the token's key head
-  __shared__ float vv[2][64 + 3];          // the value slice, then g, beta and k . q
-  __shared__ float red[2][4][2][64];
+  constexpr int DP = NW * DPW, NTH = NW * 64, ROW = 2 * DP + 68;      // per token in LDS: k | q of the key head, the value slice, g, beta, k . q, pad
+  constexpr int CH = DPW >= 64 ? 8 : 16;               // tokens per staged chunk
+  constexpr int NPER = (CH * ROW + NTH - 1) / NTH;
+  __shared__ __attribute__((aligned(16))) float stage[2][CH][ROW];
+  __shared__ float red[2][NW][2][64];
   const int VS = (c.vdim + 63) / 64;
   const int vs = blockIdx.x % VS, h = (blockIdx.x / VS) % c.heads, b = blockIdx.x / (VS * c.heads);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -240,58 +244,81 @@ __global__ void __launch_bounds__(256) delta_fwd_kernel(ktx_delta_config c, cons
     const int d = wave * DPW + r;
     S[r] = (carried && d < D && col < V) ? Sp[(size_t)d * V + col] : 0.f;
   }
-  // the next token's inputs travel global -> registers (fetch, issued a whole token ahead so that the memory latency is off the
-  // sequential path) -> LDS (commit, into the buffer the token after the current one reads)
-  constexpr int NKQ = (2 * DP + 255) / 256;
-  float pre_kq[NKQ], pre_misc = 0.f;
-  auto fetch = [&](int t) {
-    const float* row = qkv + (size_t)t * C;
+  // The inputs of CH tokens travel global -> registers (fetch, issued a whole chunk ahead: a memory round trip takes about as long as
+  // one token's step, so it must not sit on the sequential path) -> LDS (commit, at the end of the chunk before the one that reads them).
+  float pre[NPER];
+  auto fetch = [&](int ch) {
+    const int tc = t0 + ch * CH;
 #pragma unroll
-    for (int i = 0; i < NKQ; i++) {
-      const int e = tid + i * 256, which = e / DP, d = e % DP;          // 0: k, 1: q
-      pre_kq[i] = (e < 2 * DP && d < D) ? row[(which ? 0 : GD) + kh * D + d] : 0.f;
+    for (int i = 0; i < NPER; i++) {
+      const int idx = tid + i * NTH, tok = idx / ROW, e = idx % ROW, t = tc + tok;
+      float v = 0.f;
+      if (idx < CH * ROW && t < t1) {
+        const float* row = qkv + (size_t)t * C;
+        if (e < 2 * DP) {
+          const int which = e / DP, d = e % DP;          // 0: k, 1: q
+          if (d < D) v = row[(which ? 0 : GD) + kh * D + d];
+        } else {
+          const int m = e - 2 * DP;
+          if (m < 64) v = (vs * 64 + m) < V ? row[2 * GD + h * V + vs * 64 + m] : 0.f;
+          else if (m < 67) v = gb[(size_t)t * NGB + (m == 64 ? h : (m == 65 ? H + h : 2 * H + kh))];
+        }
+      }
+      pre[i] = v;
     }
-    if (tid < 64) pre_misc = (vs * 64 + tid) < V ? row[2 * GD + h * V + vs * 64 + tid] : 0.f;
-    else if (tid == 64) pre_misc = gb[(size_t)t * NGB + h];
-    else if (tid == 65) pre_misc = gb[(size_t)t * NGB + H + h];
-    else if (tid == 66) pre_misc = gb[(size_t)t * NGB + 2 * H + kh];
   };
-  auto commit = [&](int par) {
+  auto commit = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < NKQ; i++) {
-      const int e = tid + i * 256;
-      if (e < 2 * DP) kq[par][e] = pre_kq[i];
+    for (int i = 0; i < NPER; i++) {
+      const int idx = tid + i * NTH;
+      if (idx < CH * ROW) (&stage[buf][0][0])[idx] = pre[i];
     }
-    if (tid < 67) vv[par][tid] = pre_misc;
   };
-  fetch(t0);
+  const int nch = (t1 - t0 + CH - 1) / CH;
+  fetch(0);
   commit(0);
-  if (t0 + 1 < t1) fetch(t0 + 1);
+  if (nch > 1) fetch(1);
   __syncthreads();
-  for (int t = t0; t < t1; t++) {
-    const int par = (t - t0) & 1;
-    const float g = vv[par][64], beta = vv[par][65], kdq = vv[par][66], val = vv[par][lane];
-    float kr[DPW];
-    float pk = 0.f, pq = 0.f;
+  for (int ch = 0; ch < nch; ch++) {
+    const int buf = ch & 1, tc = t0 + ch * CH, n = min(CH, t1 - tc);
+    for (int i = 0; i < n; i++) {
+      const int par = i & 1, t = tc + i;
+      const float* kq = stage[buf][i];
+      const float g = kq[2 * DP + 64], beta = kq[2 * DP + 65], kdq = kq[2 * DP + 66], val = kq[2 * DP + lane];
+      float kr[DPW];
+      float pk = 0.f, pq = 0.f, pk1 = 0.f, pq1 = 0.f;
+      const float4* k4p = reinterpret_cast<const float4*>(kq + wave * DPW);       // 16-byte LDS reads, the same address in every lane
+      const float4* q4p = reinterpret_cast<const float4*>(kq + DP + wave * DPW);
 #pragma unroll
-    for (int r = 0; r < DPW; r++) {
-      const float kd = kq[par][wave * DPW + r], qd = kq[par][DP + wave * DPW + r];
-      kr[r] = kd;
-      S[r] *= g;
-      pk = fmaf(kd, S[r], pk);
-      pq = fmaf(qd, S[r], pq);
+      for (int r4 = 0; r4 < DPW / 4; r4++) {
+        const float4 k4 = k4p[r4], q4 = q4p[r4];
+        const int r = r4 * 4;
+        kr[r] = k4.x; kr[r + 1] = k4.y; kr[r + 2] = k4.z; kr[r + 3] = k4.w;
+        S[r] *= g; S[r + 1] *= g; S[r + 2] *= g; S[r + 3] *= g;
+        pk = fmaf(k4.x, S[r], pk); pk1 = fmaf(k4.y, S[r + 1], pk1); pk = fmaf(k4.z, S[r + 2], pk); pk1 = fmaf(k4.w, S[r + 3], pk1);
+        pq = fmaf(q4.x, S[r], pq); pq1 = fmaf(q4.y, S[r + 1], pq1); pq = fmaf(q4.z, S[r + 2], pq); pq1 = fmaf(q4.w, S[r + 3], pq1);
+      }
+      pk += pk1;
+      pq += pq1;
+      red[par][wave][0][lane] = pk;
+      red[par][wave][1][lane] = pq;
+      lds_barrier();
+      float kS = 0.f, qS = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; w++) {
+        kS += red[par][w][0][lane];
+        qS += red[par][w][1][lane];
+      }
+      const float u = beta * (val - kS);
+#pragma unroll
+      for (int r = 0; r < DPW; r++) S[r] = fmaf(kr[r], u, S[r]);
+      if (wave == 0 && col < V) o[((size_t)t * H + h) * V + col] = fmaf(u, kdq, qS);
     }
-    red[par][wave][0][lane] = pk;
-    red[par][wave][1][lane] = pq;
-    if (t + 1 < t1) commit(par ^ 1);
-    if (t + 2 < t1) fetch(t + 2);
-    __syncthreads();
-    const float kS = (red[par][0][0][lane] + red[par][1][0][lane]) + (red[par][2][0][lane] + red[par][3][0][lane]);
-    const float qS = (red[par][0][1][lane] + red[par][1][1][lane]) + (red[par][2][1][lane] + red[par][3][1][lane]);
-    const float u = beta * (val - kS);
-#pragma unroll
-    for (int r = 0; r < DPW; r++) S[r] = fmaf(kr[r], u, S[r]);
-    if (wave == 0 && col < V) o[((size_t)t * H + h) * V + col] = fmaf(u, kdq, qS);
+    if (ch + 1 < nch) {
+      commit(buf ^ 1);          // (every wavefront has passed the last barrier of chunk ch - 1, whose tokens this buffer held)
+      if (ch + 2 < nch) fetch(ch + 2);
+      lds_barrier();
+    }
   }
 #pragma unroll
   for (int r = 0; r < DPW; r++) {
@@ -1023,13 +1050,14 @@ int ktx_delta_forward(const ktx_delta_config* cfg, int B, const int32_t* d_q_ind
   if (B == 0) return 0;
   const unsigned blocks = (unsigned)B * cfg->heads * ((cfg->vdim + 63) / 64);
   hipStream_t st = (hipStream_t)stream;
-  const int dpw = (cfg->dim + 3) / 4;
-#define KTX_DL_GO(DPW) delta_fwd_kernel<DPW><<<blocks, 256, 0, st>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_qkv, d_gb, d_S, d_o)
-  if (dpw <= 4) KTX_DL_GO(4);
-  else if (dpw <= 8) KTX_DL_GO(8);
-  else if (dpw <= 16) KTX_DL_GO(16);
-  else if (dpw <= 32) KTX_DL_GO(32);
-  else KTX_DL_GO(64);
+  // eight wavefronts per workgroup once a quarter of the rows is more than 8: the per-token step is bound by a wavefront's rows
+#define KTX_DL_GO(DPW, NW) delta_fwd_kernel<DPW, NW><<<blocks, NW * 64, 0, st>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_qkv, d_gb, d_S, d_o)
+  const int D = cfg->dim;
+  if (D <= 16) KTX_DL_GO(4, 4);
+  else if (D <= 32) KTX_DL_GO(8, 4);
+  else if (D <= 64) KTX_DL_GO(8, 8);
+  else if (D <= 128) KTX_DL_GO(16, 8);
+  else KTX_DL_GO(32, 8);
 #undef KTX_DL_GO
   KTX_HIP(hipGetLastError());
   return 0;
