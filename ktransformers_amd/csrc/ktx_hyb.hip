@@ -157,12 +157,27 @@ __global__ void __launch_bounds__(256) delta_prep_kernel(ktx_delta_config c, con
   for (int e = tid; e < C; e += 256) {
     const int col = e < GD ? q_off + e : (e < 2 * GD ? k_off + e - GD : v_off + e - 2 * GD);
     float acc = 0.f;
-    for (int j = 0; j < K; j++) {          // input i - j times the tap K - 1 - j
-      const int ii = i - j;
-      float v = 0.f;
-      if (ii >= 0) v = proj[(size_t)(first + ii) * ldp + col];
-      else if (carried) v = st[(size_t)(K - 1 + ii) * C + e];
-      acc += taps[(size_t)e * K + (K - 1 - j)] * v;
+    if (K <= 8) {                          // every load from an address that is always valid, so that none waits for another
+      float v[8], w[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const int jj = j < K ? j : 0, ii = i - jj;
+        const bool live = j < K && (ii >= 0 || carried);
+        const float* src = ii >= 0 ? proj + (size_t)(first + ii) * ldp + col : (carried ? st + (size_t)(K - 1 + ii) * C + e : taps);
+        v[j] = *src;
+        w[j] = taps[(size_t)e * K + (K - 1 - jj)];
+        if (!live) v[j] = 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; j++) acc += w[j] * v[j];
+    } else {
+      for (int j = 0; j < K; j++) {        // input i - j times the tap K - 1 - j
+        const int ii = i - j;
+        float v = 0.f;
+        if (ii >= 0) v = proj[(size_t)(first + ii) * ldp + col];
+        else if (carried) v = st[(size_t)(K - 1 + ii) * C + e];
+        acc += taps[(size_t)e * K + (K - 1 - j)] * v;
+      }
     }
     ch[e] = silu_f32(acc);
   }
@@ -479,29 +494,36 @@ __global__ void __launch_bounds__(256) latattn_fwd_kernel(ktx_latattn_config c, 
   }
 }
 
-// merge the key ranges of one (token, head): thread = latent entry
+// merge the key ranges of one (token, head): thread = latent entry; the ranges' (maximum, sum) pairs are fetched in parallel first
 template <typename OT>
 __global__ void __launch_bounds__(256) latattn_merge_kernel(int T, int H, int L, int nsplit, const float* __restrict__ scratch,
                                                             const float* __restrict__ sink, OT* __restrict__ out) {
+  extern __shared__ float mw[];            // [nsplit] maxima, then [nsplit] weights exp(m_z - M) (0 for an empty range)
+  float* ws = mw + nsplit;
   const int t = blockIdx.x, h = blockIdx.y;
   const float sk = sink[h];
-  float M = sk;
-  for (int z = 0; z < nsplit; z++) M = fmaxf(M, scratch[(((size_t)z * T + t) * H + h) * (L + 2) + L]);
-  float den = expf(sk - M);
-  for (int z = 0; z < nsplit; z++) {
-    const float* part = scratch + (((size_t)z * T + t) * H + h) * (L + 2);
-    if (part[L] != -INFINITY) den += part[L + 1] * expf(part[L] - M);
+  const size_t stride = (size_t)T * H * (L + 2);
+  const float* base = scratch + ((size_t)t * H + h) * (L + 2);
+  for (int z = threadIdx.x; z < nsplit; z += 256) {
+    mw[z] = base[z * stride + L];
+    ws[z] = base[z * stride + L + 1];
   }
+  __syncthreads();
+  float M = sk;
+  for (int z = 0; z < nsplit; z++) M = fmaxf(M, mw[z]);
+  float den = expf(sk - M);
+  for (int z = 0; z < nsplit; z++) den += mw[z] == -INFINITY ? 0.f : ws[z] * expf(mw[z] - M);
+  __syncthreads();
+  for (int z = threadIdx.x; z < nsplit; z += 256) ws[z] = mw[z] == -INFINITY ? 0.f : expf(mw[z] - M);
+  __syncthreads();
+  const float inv = 1.0f / den;
   for (int l = threadIdx.x; l < L; l += 256) {
     float a = 0.f;
-    for (int z = 0; z < nsplit; z++) {
-      const float* part = scratch + (((size_t)z * T + t) * H + h) * (L + 2);
-      if (part[L] != -INFINITY) a += part[l] * expf(part[L] - M);
-    }
-    st_elem(out, ((size_t)t * H + h) * L + l, a / den);
+#pragma unroll 4
+    for (int z = 0; z < nsplit; z++) a = fmaf(base[z * stride + l], ws[z], a);
+    st_elem(out, ((size_t)t * H + h) * L + l, a * inv);
   }
 }
-
 
 // The same attention on the matrix cores (bf16 latent cache).  The latent rows are keys AND values of every head, so the (token, head)
 // pairs of a request are the rows of one long query matrix against shared keys: a workgroup takes 64 consecutive rows (its four
@@ -538,14 +560,22 @@ __global__ void __launch_bounds__(256) latattn_mfma_kernel(ktx_latattn_config c,
   sq_v8bf qf[KSMAX];
   {
     const int ar = rw0 + l16;
-    const float* qrow = q + ((size_t)t0 * H + ar) * E;
+    const bool live = ar < rows_total;
+    const float* qrow = q + ((size_t)t0 * H + (live ? ar : rows_total - 1)) * E;       // (E % 8 == 0: 16-byte pieces stay inside the row)
 #pragma unroll
     for (int kk = 0; kk < KSMAX; kk++) {
       float v[8];
+      const int e0 = kk * 32 + lq * 8;
+      if (kk < KS && e0 < E) {
+        const float4 x = *reinterpret_cast<const float4*>(qrow + e0), y = *reinterpret_cast<const float4*>(qrow + e0 + 4);
+        v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w; v[4] = y.x; v[5] = y.y; v[6] = y.z; v[7] = y.w;
+      } else {
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        const int e = kk * 32 + lq * 8 + i;
-        v[i] = (kk < KS && ar < rows_total && e < E) ? qrow[e] : 0.f;
+        for (int i = 0; i < 8; i++) v[i] = 0.f;
+      }
+      if (!live) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = 0.f;
       }
       union { uint4 u; sq_v8bf f; } cv;
       cv.u.x = ktx_pk_bf16(v[0], v[1]); cv.u.y = ktx_pk_bf16(v[2], v[3]); cv.u.z = ktx_pk_bf16(v[4], v[5]); cv.u.w = ktx_pk_bf16(v[6], v[7]);
@@ -1093,7 +1123,7 @@ int ktx_latattn_forward(const ktx_latattn_config* cfg, int T, const float* d_q, 
   if (latattn_check(cfg, "ktx_latattn_forward")) return -1;
   KTX_REQUIRE(T >= 0 && d_q && d_cache && d_tok_req && d_pos && d_page_indptr && d_page_indices && d_sink && d_out && dtype_ok(out_dtype),
               "ktx_latattn_forward: null pointer");
-  KTX_REQUIRE(nsplit >= 1 && nsplit <= 65535 && (nsplit == 1 || d_scratch), "ktx_latattn_forward: nsplit >= 1, scratch when > 1");
+  KTX_REQUIRE(nsplit >= 1 && nsplit <= 4096 && (nsplit == 1 || d_scratch), "ktx_latattn_forward: 1 <= nsplit <= 4096, scratch when > 1");
   if (T == 0) return 0;
   const int L = cfg->kv_rank, E = L + cfg->rot_dim;
   KTX_REQUIRE(L <= 256 * LA_NACC, "ktx_latattn_forward: kv_rank <= 8192");
@@ -1125,8 +1155,8 @@ int ktx_latattn_forward(const ktx_latattn_config* cfg, int T, const float* d_q, 
   KTX_HIP(hipGetLastError());
   if (nsplit > 1) {
     const dim3 mg(T, cfg->heads);
-    if (out_dtype == KTX_SEQ_F32) latattn_merge_kernel<float><<<mg, 256, 0, st>>>(T, cfg->heads, L, nsplit, d_scratch, d_sink, (float*)d_out);
-    else latattn_merge_kernel<bf16_t><<<mg, 256, 0, st>>>(T, cfg->heads, L, nsplit, d_scratch, d_sink, (bf16_t*)d_out);
+    if (out_dtype == KTX_SEQ_F32) latattn_merge_kernel<float><<<mg, 256, (size_t)nsplit * 8, st>>>(T, cfg->heads, L, nsplit, d_scratch, d_sink, (float*)d_out);
+    else latattn_merge_kernel<bf16_t><<<mg, 256, (size_t)nsplit * 8, st>>>(T, cfg->heads, L, nsplit, d_scratch, d_sink, (bf16_t*)d_out);
     KTX_HIP(hipGetLastError());
   }
   return 0;
@@ -1148,7 +1178,7 @@ int ktx_latattn_mfma(const ktx_latattn_config* cfg, int B, int T, int max_q_len,
   KTX_REQUIRE(B >= 0 && T >= 0 && max_q_len >= 0 && d_q && d_cache && d_q_indptr && d_pos0 && d_page_indptr && d_page_indices && d_sink &&
                   d_out && dtype_ok(out_dtype),
               "ktx_latattn_mfma: null pointer");
-  KTX_REQUIRE(nsplit >= 1 && nsplit <= 65535 && (nsplit == 1 || d_scratch), "ktx_latattn_mfma: nsplit >= 1, scratch when > 1");
+  KTX_REQUIRE(nsplit >= 1 && nsplit <= 4096 && (nsplit == 1 || d_scratch), "ktx_latattn_mfma: 1 <= nsplit <= 4096, scratch when > 1");
   if (B == 0 || T == 0 || max_q_len == 0) return 0;
   const int row_tiles = (int)(((int64_t)max_q_len * cfg->heads + 63) / 64);
   const dim3 grid((unsigned)B * row_tiles, 1, nsplit);
@@ -1175,8 +1205,8 @@ int ktx_latattn_mfma(const ktx_latattn_config* cfg, int B, int T, int max_q_len,
   KTX_HIP(hipGetLastError());
   if (nsplit > 1) {
     const dim3 mg(T, cfg->heads);
-    if (out_dtype == KTX_SEQ_F32) latattn_merge_kernel<float><<<mg, 256, 0, st>>>(T, cfg->heads, L, nsplit, d_scratch, d_sink, (float*)d_out);
-    else latattn_merge_kernel<bf16_t><<<mg, 256, 0, st>>>(T, cfg->heads, L, nsplit, d_scratch, d_sink, (bf16_t*)d_out);
+    if (out_dtype == KTX_SEQ_F32) latattn_merge_kernel<float><<<mg, 256, (size_t)nsplit * 8, st>>>(T, cfg->heads, L, nsplit, d_scratch, d_sink, (float*)d_out);
+    else latattn_merge_kernel<bf16_t><<<mg, 256, (size_t)nsplit * 8, st>>>(T, cfg->heads, L, nsplit, d_scratch, d_sink, (bf16_t*)d_out);
     KTX_HIP(hipGetLastError());
   }
   return 0;
