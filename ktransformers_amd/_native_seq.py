@@ -32,7 +32,9 @@ class _MlstmConfig(C.Structure):     # include/ktx_seq.h: ktx_mlstm_config
 
 
 def _load() -> C.CDLL:
-    path = next((p for p in LIB_PATHS if os.path.exists(p)), None)
+    have = [p for p in LIB_PATHS if os.path.exists(p)]
+    # the whole library when it is there — unless the subset library was built after it (sources changed and only the subset was rebuilt)
+    path = max(have, key=os.path.getmtime) if len(have) == 2 and os.path.getmtime(have[1]) > os.path.getmtime(have[0]) else (have[0] if have else None)
     if path is None:
         raise ImportError(f"neither {LIB_PATHS[0]} nor {LIB_PATHS[1]} found: build with `python -m ktransformers_amd.build [--seq]` "
                           "(hipcc, gfx950).  ktransformers_amd has no CPU fallback.")
