@@ -123,17 +123,18 @@ int ktx_moe_plan(int T, int E, int top, int tile_m, const int32_t* d_topk_idx, i
                  int32_t* d_pair_pos, int32_t* d_sorted_group, int32_t* d_tile_group, int32_t* d_tile_row0, int32_t* d_num_tiles,
                  ktx_stream_t stream);
 
-enum { KTX_GG_TILE_M = 64 };
+enum { KTX_GG_TILE_M = 64, KTX_GG_TILE_M_WIDE = 128 };
 
 /* Grouped GEMM  Y_g = A_g W_g^T  on the matrix cores (the product runs in W's type like ktx_dense_gemm; Y fp32 or bf16).
  * W: G matrices [N][K] back to back.
  * Uniform form (d_group_off NULL): every group g < G multiplies the same M rows; A_g = columns a_goff * g .. of A's rows, Y_g = columns
  *   y_goff * g .. of Y's rows (per-head products of a [T][heads][.] tensor).
  * Ragged form: sorted rows group_off[g] .. group_off[g+1] belong to group g; the A row of sorted row r is a_rows[r] (NULL: r itself), its
- *   Y row is r; tiles come from ktx_moe_plan (max_tiles bounds the launch, num_tiles[0] on the device says how many are real). */
+ *   Y row is r; tiles come from ktx_moe_plan (max_tiles bounds the launch, num_tiles[0] on the device says how many are real) and hold
+ *   tile_m = 64 rows, or 128 (bf16 products only: the wide tile prompts take). */
 int ktx_grouped_gemm(int G, int M, int N, int K, const void* d_A, int a_dtype, int64_t lda, int64_t a_goff, const int32_t* d_a_rows,
                      const void* d_W, int w_dtype, void* d_Y, int y_dtype, int64_t ldy, int64_t y_goff, const int32_t* d_group_off,
-                     const int32_t* d_tile_group, const int32_t* d_tile_row0, const int32_t* d_num_tiles, int max_tiles,
+                     const int32_t* d_tile_group, const int32_t* d_tile_row0, const int32_t* d_num_tiles, int max_tiles, int tile_m,
                      ktx_stream_t stream);
 
 /* The ragged products for a handful of rows (decode steps), streaming each row's weights once: Y[r] = W_g A[a_rows ? a_rows[r] : r]

@@ -40,9 +40,10 @@ lib.ktx_latattn_mfma.argtypes = [C.POINTER(_LatAttnConfig), _I, _I, _I, _P, _P, 
 lib.ktx_moe_route.argtypes = [_I, _I, _I, _F, _F, _P, _L, _P, _P, _P]
 lib.ktx_moe_plan.argtypes = [_I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P]
 lib.ktx_grouped_gemv.argtypes = [_I, _I, _I, _P, _I, _L, _P, _P, _I, _P, _I, _L, _P, _I, _P]
-lib.ktx_grouped_gemm.argtypes = [_I, _I, _I, _I, _P, _I, _L, _L, _P, _P, _I, _P, _I, _L, _L, _P, _P, _P, _P, _I, _P]
+lib.ktx_grouped_gemm.argtypes = [_I, _I, _I, _I, _P, _I, _L, _L, _P, _P, _I, _P, _I, _L, _L, _P, _P, _P, _P, _I, _I, _P]
 
 TILE_M = 64
+TILE_M_WIDE, WIDE_MIN_ROWS_PER_EXPERT = 128, 96      # bf16 steps whose experts average this many rows take 128-row tiles
 
 
 def _ptr(t):
@@ -239,22 +240,24 @@ def moe_route(logits: torch.Tensor, top: int, scale: float, sum_eps: float):
 
 
 class MoePlan:
-    __slots__ = ("group_off", "sorted_tok", "pair_pos", "sorted_group", "tile_group", "tile_row0", "num_tiles", "max_tiles", "pairs")
+    __slots__ = ("group_off", "sorted_tok", "pair_pos", "sorted_group", "tile_group", "tile_row0", "num_tiles", "max_tiles", "pairs", "tile_m")
 
 
-def moe_plan(topk_idx: torch.Tensor, E: int) -> MoePlan:
+def moe_plan(topk_idx: torch.Tensor, E: int, wide: bool = False) -> MoePlan:
+    """Sort the pairs by expert and lay the row tiles out (ktx_moe_plan).  wide: 128-row tiles (bf16 products of prompt-sized steps)."""
     _i32(topk_idx, "moe_plan topk_idx")
     T, top = topk_idx.shape
     p = MoePlan()
     p.pairs = T * top
-    p.max_tiles = p.pairs // TILE_M + min(E, p.pairs) + 1
+    p.tile_m = TILE_M_WIDE if wide else TILE_M
+    p.max_tiles = p.pairs // p.tile_m + min(E, p.pairs) + 1
     meta = torch.empty(E + 1 + 3 * p.pairs + 2 * p.max_tiles + 1, dtype=torch.int32, device=topk_idx.device)
     at = 0
     for name, n in (("group_off", E + 1), ("sorted_tok", p.pairs), ("pair_pos", p.pairs), ("sorted_group", p.pairs), ("tile_group", p.max_tiles),
                     ("tile_row0", p.max_tiles), ("num_tiles", 1)):
         setattr(p, name, meta[at:at + n])
         at += n
-    check(lib.ktx_moe_plan(T, E, top, TILE_M, topk_idx.data_ptr(), p.group_off.data_ptr(), p.sorted_tok.data_ptr(), p.pair_pos.data_ptr(),
+    check(lib.ktx_moe_plan(T, E, top, p.tile_m, topk_idx.data_ptr(), p.group_off.data_ptr(), p.sorted_tok.data_ptr(), p.pair_pos.data_ptr(),
                            p.sorted_group.data_ptr(), p.tile_group.data_ptr(), p.tile_row0.data_ptr(), p.num_tiles.data_ptr(), _stream_ptr(topk_idx.device)))
     return p
 
@@ -273,7 +276,7 @@ def head_gemm(a: torch.Tensor, a_goff: int, w: torch.Tensor, out: torch.Tensor, 
     _gg_types(a, w, out.dtype)
     M = a.shape[0]
     check(lib.ktx_grouped_gemm(G, M, N, K, a.data_ptr(), SEQ_DTYPE[a.dtype], a.stride(0), a_goff, None, w.data_ptr(), SEQ_DTYPE[w.dtype],
-                               out.data_ptr(), SEQ_DTYPE[out.dtype], out.stride(0), y_goff, None, None, None, None, 0, _stream_ptr(a.device)))
+                               out.data_ptr(), SEQ_DTYPE[out.dtype], out.stride(0), y_goff, None, None, None, None, 0, TILE_M, _stream_ptr(a.device)))
     return out
 
 
@@ -298,5 +301,5 @@ def expert_gemm(a: torch.Tensor, w: torch.Tensor, plan: MoePlan, gather: bool, o
     check(lib.ktx_grouped_gemm(G, plan.pairs, N, K, a.data_ptr(), SEQ_DTYPE[a.dtype], a.stride(0), 0,
                                plan.sorted_tok.data_ptr() if gather else None, w.data_ptr(), SEQ_DTYPE[w.dtype], out.data_ptr(),
                                SEQ_DTYPE[out_dtype], out.stride(0), 0, plan.group_off.data_ptr(), plan.tile_group.data_ptr(),
-                               plan.tile_row0.data_ptr(), plan.num_tiles.data_ptr(), plan.max_tiles, _stream_ptr(a.device)))
+                               plan.tile_row0.data_ptr(), plan.num_tiles.data_ptr(), plan.max_tiles, plan.tile_m, _stream_ptr(a.device)))
     return out

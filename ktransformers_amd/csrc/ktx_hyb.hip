@@ -901,6 +901,58 @@ __global__ void __launch_bounds__(256) grouped_gemm_kernel(int M, int N, int K, 
       }
 }
 
+// the ragged form for prompts: a 128 x 128 x 32 tile (bf16 MFMA), four wavefronts of 64 x 64 = 4 x 4 MFMA tiles — four times the
+// products per LDS fragment read of the 64 x 64 tile; tiles of 128 sorted rows come from ktx_moe_plan(tile_m = 128)
+template <typename AT, typename YT>
+__global__ void __launch_bounds__(256) grouped_gemm128_kernel(int N, int K, const AT* __restrict__ A, int64_t lda,
+                                                              const int32_t* __restrict__ a_rows, const bf16_t* __restrict__ W,
+                                                              YT* __restrict__ Y, int64_t ldy, const int32_t* __restrict__ group_off,
+                                                              const int32_t* __restrict__ tile_group, const int32_t* __restrict__ tile_row0,
+                                                              const int32_t* __restrict__ num_tiles, bool vec_a, bool vec_w) {
+  constexpr int LD = GemmTraits<bf16_t>::LDS_LD;
+  __shared__ __attribute__((aligned(16))) bf16_t As[128 * LD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[128 * LD];
+  if ((int)blockIdx.y >= num_tiles[0]) return;
+  const int g = tile_group[blockIdx.y], m0 = tile_row0[blockIdx.y], m_end = group_off[g + 1];
+  const bf16_t* Wg = W + (size_t)g * N * K;
+  const int n0 = blockIdx.x * 128;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int l16 = lane & 15, lq = lane >> 4;
+  v4f acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    __syncthreads();
+    gg_stage_rows<AT, bf16_t>(As, A, lda, a_rows, m0, m_end, k0, K, vec_a);
+    gg_stage_rows<AT, bf16_t>(As + 64 * LD, A, lda, a_rows, m0 + 64, m_end, k0, K, vec_a);
+    gemm_stage<bf16_t, bf16_t>(Ws, Wg, (int64_t)K, n0, N, k0, K, vec_w);
+    gemm_stage<bf16_t, bf16_t>(Ws + 64 * LD, Wg, (int64_t)K, n0 + 64, N, k0, K, vec_w);
+    __syncthreads();
+    sq_v8bf af[4], bf[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      af[i] = *reinterpret_cast<const sq_v8bf*>(As + (wm + i * 16 + l16) * LD + lq * 8);
+      bf[i] = *reinterpret_cast<const sq_v8bf*>(Ws + (wn + i * 16 + l16) * LD + lq * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int m = m0 + wm + i * 16 + lq * 4 + r, n = n0 + wn + j * 16 + l16;
+        if (m < m_end && n < N) st_elem(Y, (size_t)m * ldy + n, acc[i][j][r]);
+      }
+}
+
 // the same products for a handful of rows (decode steps): no tile, the weights stream once per row.  Workgroup = (8 output columns,
 // one sorted row); a wavefront owns two columns and its lanes stride over K in 16-byte pieces.  glu: column f pairs rows f and
 // F + f of the group's [2F][K] matrix and writes silu(first) * second.
@@ -1237,7 +1289,7 @@ int ktx_moe_plan(int T, int E, int top, int tile_m, const int32_t* d_topk_idx, i
 
 int ktx_grouped_gemm(int G, int M, int N, int K, const void* d_A, int a_dtype, int64_t lda, int64_t a_goff, const int32_t* d_a_rows,
                      const void* d_W, int w_dtype, void* d_Y, int y_dtype, int64_t ldy, int64_t y_goff, const int32_t* d_group_off,
-                     const int32_t* d_tile_group, const int32_t* d_tile_row0, const int32_t* d_num_tiles, int max_tiles,
+                     const int32_t* d_tile_group, const int32_t* d_tile_row0, const int32_t* d_num_tiles, int max_tiles, int tile_m,
                      ktx_stream_t stream) {
   KTX_REQUIRE(G > 0 && M >= 0 && N > 0 && K > 0 && d_A && d_W && d_Y, "ktx_grouped_gemm: G, N, K > 0, pointers");
   KTX_REQUIRE(dtype_ok(a_dtype) && dtype_ok(w_dtype) && dtype_ok(y_dtype), "ktx_grouped_gemm: unknown element type");
@@ -1248,6 +1300,26 @@ int ktx_grouped_gemm(int G, int M, int N, int K, const void* d_A, int a_dtype, i
   KTX_REQUIRE(ragged || (G <= 65535 && !d_a_rows), "ktx_grouped_gemm: the uniform form takes up to 65535 groups and no gather");
   const int ytiles = ragged ? max_tiles : (M + 63) / 64;
   if (ytiles == 0) return 0;
+  if (ragged && tile_m == 128) {
+    KTX_REQUIRE(w_dtype == KTX_SEQ_BF16, "ktx_grouped_gemm: 128-row tiles are the bf16 product's");
+    KTX_REQUIRE(ytiles <= 65535, "ktx_grouped_gemm: too many row tiles");
+    const dim3 grid128((N + 127) / 128, ytiles, 1);
+    const size_t asz1 = a_dtype == KTX_SEQ_F32 ? 4 : 2;
+    const bool va = aligned16(d_A) && (lda * asz1) % 16 == 0 && K % 8 == 0;
+    const bool vw = aligned16(d_W) && ((size_t)K * 2) % 16 == 0 && K % 8 == 0 && ((size_t)N * K * 2) % 16 == 0;
+    hipStream_t st1 = (hipStream_t)stream;
+#define KTX_GG128_GO(AT, YT)                                                                                                       \
+  grouped_gemm128_kernel<AT, YT><<<grid128, 256, 0, st1>>>(N, K, (const AT*)d_A, lda, d_a_rows, (const bf16_t*)d_W, (YT*)d_Y, ldy, \
+                                                           d_group_off, d_tile_group, d_tile_row0, d_num_tiles, va, vw)
+    if (a_dtype == KTX_SEQ_F32 && y_dtype == KTX_SEQ_F32) KTX_GG128_GO(float, float);
+    else if (a_dtype == KTX_SEQ_F32) KTX_GG128_GO(float, bf16_t);
+    else if (y_dtype == KTX_SEQ_F32) KTX_GG128_GO(bf16_t, float);
+    else KTX_GG128_GO(bf16_t, bf16_t);
+#undef KTX_GG128_GO
+    KTX_HIP(hipGetLastError());
+    return 0;
+  }
+  KTX_REQUIRE(!ragged || tile_m == 64, "ktx_grouped_gemm: tiles of 64 or 128 rows");
   KTX_REQUIRE(ytiles <= 65535, "ktx_grouped_gemm: too many row tiles");
   const dim3 grid((N + 63) / 64, ytiles, ragged ? 1 : G);
   const size_t asz = a_dtype == KTX_SEQ_F32 ? 4 : 2, wsz = w_dtype == KTX_SEQ_F32 ? 4 : 2;

@@ -52,7 +52,7 @@ class KSigmoidRoutedMoE(BaseInjectedModule):
     def forward(self, h: torch.Tensor, rider=None):
         """h [T, width] in the compute type -> (shared expert's output fp32 [T, width] or None, the rider's product or None,
         expert_rows fp32 [T * top, width] in sorted order, pair_pos int32 [T * top], topk_w fp32 [T, top])."""
-        from ktransformers_amd._native_hyb import GEMV_MAX_ROWS, expert_gemm, moe_plan, moe_route, silu_mul_rows
+        from ktransformers_amd._native_hyb import GEMV_MAX_ROWS, WIDE_MIN_ROWS_PER_EXPERT, expert_gemm, moe_plan, moe_route, silu_mul_rows
         from ktransformers_amd._native_seq import dense_gemm
         k = id(rider) if rider is not None else None
         if k not in self._merged:
@@ -61,7 +61,8 @@ class KSigmoidRoutedMoE(BaseInjectedModule):
         E, SF = self.experts, self.shared_ff or 0
         proj = dense_gemm(h, self._merged[k])
         idx, wts = moe_route(proj[:, :E], self.top, self.route_scale, self.sum_eps)
-        plan = moe_plan(idx, E)
+        wide = self.compute_dtype == torch.bfloat16 and h.shape[0] * self.top >= WIDE_MIN_ROWS_PER_EXPERT * E
+        plan = moe_plan(idx, E, wide=wide)
         if plan.pairs <= GEMV_MAX_ROWS:      # decode steps: the weights stream once per pair, the activation in the same launch
             act = expert_gemm(h, self.w["gate_up"], plan, gather=True, out_dtype=self.compute_dtype, glu=True)
         else:

@@ -178,6 +178,12 @@ def test_router_and_expert_sort(E, top, T):
     tiles = list(zip(plan.tile_group.cpu().tolist()[:nt], plan.tile_row0.cpu().tolist()[:nt]))
     want = [(e, r) for e in range(E) for r in range(off[e], off[e + 1], 64)]
     assert tiles == want and nt <= plan.max_tiles
+    assert plan.sorted_group.cpu().tolist() == [e for e in range(E) for _ in range(off[e], off[e + 1])]
+    wide = moe_plan(idx, E, wide=True)          # 128-row tiles (what prompt-sized bf16 steps take)
+    off = wide.group_off.cpu().tolist()
+    nt = int(wide.num_tiles.cpu())
+    assert list(zip(wide.tile_group.cpu().tolist()[:nt], wide.tile_row0.cpu().tolist()[:nt])) == \
+        [(e, r) for e in range(E) for r in range(off[e], off[e + 1], 128)] and nt <= wide.max_tiles
 
 
 def _operator(cfg, seed, dtype, page_size=8, P=None):
@@ -305,7 +311,8 @@ def test_one_key_at_the_window_edge_stands_out(dtype, window, query, back, L):
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
-@pytest.mark.parametrize("E,top,F,SF,T", [(6, 2, 24, 24, 50), (3, 1, 7, 0, 9), (4, 4, 32, 64, 130), (16, 3, 40, 8, 1)])
+@pytest.mark.parametrize("E,top,F,SF,T", [(6, 2, 24, 24, 50), (3, 1, 7, 0, 9), (4, 4, 32, 64, 130), (16, 3, 40, 8, 1), (3, 2, 136, 16, 400),
+                                          (5, 2, 20, 0, 333)])
 def test_mixture_of_experts(dtype, E, top, F, SF, T):
     cfg = R.make_config([R.delta_layer(mlp=R.moe_mlp(experts=E, top=top, ff=F, shared_ff=SF, scale=1.3))], width=40)
     model, cache, P = build(cfg, 4, dtype)
