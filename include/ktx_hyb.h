@@ -30,10 +30,13 @@ int ktx_layer_norm(int T, int W, const float* d_x, const float* d_w, const float
  *   z[t] = (y ? y[t] : 0) + (ybias ? ybias : 0) + sum_{k < top} topk_w[t][k] * ey[pair_pos[t * top + k]]     (ey NULL: no such term)
  *   z   *= sigmoid(gl[t] + gbias)                                                                            (gl NULL: no gate)
  *   x[t] += layer_norm(z; wn, bn, eps)
- * y fp32 rows of stride ldy, ey fp32 [pairs][W], gl fp32 rows of stride ldg, all vectors fp32 [W]; x fp32 [T][W] in place. */
+ *   next_out[t] = layer_norm(x[t]; next_w, next_b, next_eps)      (next_w NULL: not written) — the pre-norm of the sublayer that follows
+ * y fp32 rows of stride ldy, ey fp32 [pairs][W], gl fp32 rows of stride ldg, all vectors fp32 [W]; x fp32 [T][W] in place;
+ * next_out [T][W] of next_dtype. */
 int ktx_gated_norm_add(int T, int W, const float* d_y, int64_t ldy, const float* d_ybias, const float* d_ey, const int32_t* d_pair_pos,
                        const float* d_topk_w, int top, const float* d_gl, int64_t ldg, const float* d_gbias, const float* d_wn,
-                       const float* d_bn, float eps, float* d_x, ktx_stream_t stream);
+                       const float* d_bn, float eps, float* d_x, const float* d_next_w, const float* d_next_b, float next_eps,
+                       void* d_next_out, int next_dtype, ktx_stream_t stream);
 
 /* PolyNorm: with u(v) = v / sqrt(mean(v^2) + eps) over a row of F values and z = in[t] + bias,
  * out[t] = c[0] u(z) + c[1] u(z^2) + c[2] u(z^3) + c[3] (powers element-wise).  in fp32 rows of stride ldz; coef fp32 [4] on the device. */

@@ -27,7 +27,7 @@ if not hasattr(lib, "ktx_grouped_gemm"):
     raise ImportError("the loaded kernel library predates include/ktx_hyb.h: rebuild with `python -m ktransformers_amd.build [--seq]`")
 lib.ktx_rows_add.argtypes = [_I, _I, _P, _P, _P, _P]
 lib.ktx_layer_norm.argtypes = [_I, _I, _P, _P, _P, _F, _P, _P, _I, _P]
-lib.ktx_gated_norm_add.argtypes = [_I, _I, _P, _L, _P, _P, _P, _P, _I, _P, _L, _P, _P, _P, _F, _P, _P]
+lib.ktx_gated_norm_add.argtypes = [_I, _I, _P, _L, _P, _P, _P, _P, _I, _P, _L, _P, _P, _P, _F, _P, _P, _P, _F, _P, _I, _P]
 lib.ktx_poly_norm.argtypes = [_I, _I, _P, _L, _P, _P, _F, _P, _I, _P]
 lib.ktx_silu_mul_rows.argtypes = [_I, _I, _P, _L, _P, _I, _P]
 lib.ktx_head_gate_norm.argtypes = [_I, _I, _I, _F, _P, _P, _L, _P, _I, _I, _P, _I, _P]
@@ -92,9 +92,10 @@ def layer_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None, eps: fl
 
 def gated_norm_add(x: torch.Tensor, wn: torch.Tensor, bn: torch.Tensor | None, eps: float, y: torch.Tensor | None = None,
                    ybias: torch.Tensor | None = None, gate_logits: torch.Tensor | None = None, gate_bias: torch.Tensor | None = None,
-                   expert_rows: torch.Tensor | None = None, pair_pos: torch.Tensor | None = None, topk_w: torch.Tensor | None = None
-                   ) -> torch.Tensor:
-    """x += layer_norm((y + ybias + sum_k topk_w[t, k] expert_rows[pair_pos[t, k]]) * sigmoid(gate_logits + gate_bias)), in place."""
+                   expert_rows: torch.Tensor | None = None, pair_pos: torch.Tensor | None = None, topk_w: torch.Tensor | None = None,
+                   next_norm: tuple | None = None):
+    """x += layer_norm((y + ybias + sum_k topk_w[t, k] expert_rows[pair_pos[t, k]]) * sigmoid(gate_logits + gate_bias)), in place.
+    next_norm = (weight, bias or None, eps, dtype): also returns layer_norm(updated x) in that type — (x, h) instead of x."""
     _f32(x, "gated_norm_add x"), _f32(wn, "wn"), _f32(bn, "bn"), _f32(ybias, "ybias"), _f32(gate_bias, "gate_bias")
     _f32(expert_rows, "expert_rows"), _i32(pair_pos, "pair_pos"), _f32(topk_w, "topk_w")
     T, W = x.shape
@@ -108,9 +109,17 @@ def gated_norm_add(x: torch.Tensor, wn: torch.Tensor, bn: torch.Tensor | None, e
         top = topk_w.shape[1]
         if expert_rows.shape[1] != W or pair_pos.numel() != T * top or topk_w.shape[0] != T:
             raise KtxError("gated_norm_add: the gathered term does not fit")
+    h, nw, nb, neps, ndt = None, None, None, 0.0, torch.float32
+    if next_norm is not None:
+        nw, nb, neps, ndt = next_norm
+        _f32(nw, "gated_norm_add next weight"), _f32(nb, "gated_norm_add next bias")
+        if nw.numel() != W or (nb is not None and nb.numel() != W):
+            raise KtxError("gated_norm_add: the following norm does not fit the row")
+        h = torch.empty((T, W), dtype=ndt, device=x.device)
     check(lib.ktx_gated_norm_add(T, W, yp, ldy, _ptr(ybias), _ptr(expert_rows), _ptr(pair_pos), _ptr(topk_w), top, gp, ldg, _ptr(gate_bias),
-                                 wn.data_ptr(), _ptr(bn), float(eps), x.data_ptr(), _stream_ptr(x.device)))
-    return x
+                                 wn.data_ptr(), _ptr(bn), float(eps), x.data_ptr(), _ptr(nw), _ptr(nb), float(neps), _ptr(h),
+                                 SEQ_DTYPE[ndt], _stream_ptr(x.device)))
+    return x if next_norm is None else (x, h)
 
 
 def poly_norm(z: torch.Tensor, bias: torch.Tensor | None, coef: torch.Tensor, eps: float, out_dtype=torch.float32) -> torch.Tensor:

@@ -55,13 +55,17 @@ __global__ void __launch_bounds__(256) layer_norm_kernel(int W, const float* __r
   for (int e = tid; e < W; e += 256) st_elem(out, (size_t)t * W + e, (a[e] - mean) * r * w[e] + (b ? b[e] : 0.f));
 }
 
-// z = (y + ybias + sum_k w_k ey[pos_k]) * sigmoid(gl + gbias); x += LN(z).  The row lives in LDS between the passes.
+// z = (y + ybias + sum_k w_k ey[pos_k]) * sigmoid(gl + gbias); x += LN(z).  The row lives in LDS between the passes.  With nw: the
+// layer norm of the UPDATED row (the next sublayer's pre-norm) is written to nout in the same launch.
+template <typename OT>
 __global__ void __launch_bounds__(256) gated_norm_add_kernel(int W, const float* __restrict__ y, int64_t ldy,
                                                              const float* __restrict__ ybias, const float* __restrict__ ey,
                                                              const int32_t* __restrict__ pair_pos, const float* __restrict__ topk_w,
                                                              int top, const float* __restrict__ gl, int64_t ldg,
                                                              const float* __restrict__ gbias, const float* __restrict__ wn,
-                                                             const float* __restrict__ bn, float eps, float* __restrict__ x) {
+                                                             const float* __restrict__ bn, float eps, float* __restrict__ x,
+                                                             const float* __restrict__ nw, const float* __restrict__ nb, float neps,
+                                                             OT* __restrict__ nout) {
   extern __shared__ float zrow[];
   __shared__ float red[4];
   const int t = blockIdx.x, tid = threadIdx.x;
@@ -85,7 +89,22 @@ __global__ void __launch_bounds__(256) gated_norm_add_kernel(int W, const float*
     q += d * d;
   }
   const float r = 1.0f / sqrtf(block_sum256(q, red) / (float)W + eps);
-  for (int e = tid; e < W; e += 256) x[(size_t)t * W + e] += (zrow[e] - mean) * r * wn[e] + (bn ? bn[e] : 0.f);
+  float s2 = 0.f;
+  for (int e = tid; e < W; e += 256) {
+    const float v = x[(size_t)t * W + e] + ((zrow[e] - mean) * r * wn[e] + (bn ? bn[e] : 0.f));
+    x[(size_t)t * W + e] = v;
+    zrow[e] = v;              // (each thread re-reads only what it wrote)
+    s2 += v;
+  }
+  if (!nw) return;
+  const float mean2 = block_sum256(s2, red) / (float)W;
+  float q2 = 0.f;
+  for (int e = tid; e < W; e += 256) {
+    const float d = zrow[e] - mean2;
+    q2 += d * d;
+  }
+  const float r2 = 1.0f / sqrtf(block_sum256(q2, red) / (float)W + neps);
+  for (int e = tid; e < W; e += 256) st_elem(nout, (size_t)t * W + e, (zrow[e] - mean2) * r2 * nw[e] + (nb ? nb[e] : 0.f));
 }
 
 template <typename OT>
@@ -230,7 +249,7 @@ __global__ void __launch_bounds__(256) delta_conv_update_kernel(ktx_delta_config
   }
 }
 
-// the recurrence: workgroup = (request, head, 64 value columns); wavefront = dim / NW rows (NW = 4 or 8), lane = value column; the state
+// the recurrence: workgroup = (request, head, 64 value columns); wavefront = dim / NW rows (NW = 4, 8 or 16), lane = value column; the state
 // slice stays in registers; ONE barrier per token: both read-outs (S^T k and S^T q of the decayed state) are taken before the write,
 // o = (g S)^T q + u (k . q).  The tokens' inputs are staged through LDS a chunk ahead.
 template <int DPW, int NW>
@@ -1047,13 +1066,20 @@ int ktx_layer_norm(int T, int W, const float* d_x, const float* d_w, const float
 
 int ktx_gated_norm_add(int T, int W, const float* d_y, int64_t ldy, const float* d_ybias, const float* d_ey, const int32_t* d_pair_pos,
                        const float* d_topk_w, int top, const float* d_gl, int64_t ldg, const float* d_gbias, const float* d_wn,
-                       const float* d_bn, float eps, float* d_x, ktx_stream_t stream) {
+                       const float* d_bn, float eps, float* d_x, const float* d_next_w, const float* d_next_b, float next_eps,
+                       void* d_next_out, int next_dtype, ktx_stream_t stream) {
   KTX_REQUIRE(T >= 0 && W > 0 && d_wn && d_x && (d_y || d_ey), "ktx_gated_norm_add: arguments");
   KTX_REQUIRE(!d_ey || (d_pair_pos && d_topk_w && top > 0), "ktx_gated_norm_add: the gathered term needs pair_pos, topk_w and top");
+  KTX_REQUIRE(!d_next_w || (d_next_out && dtype_ok(next_dtype)), "ktx_gated_norm_add: the following norm needs its output");
   KTX_REQUIRE((size_t)W * 4 <= 64 * 1024, "ktx_gated_norm_add: rows up to 16384 entries");
   if (T == 0) return 0;
-  gated_norm_add_kernel<<<T, 256, (size_t)W * 4, (hipStream_t)stream>>>(W, d_y, ldy, d_ybias, d_ey, d_pair_pos, d_topk_w, top, d_gl, ldg,
-                                                                          d_gbias, d_wn, d_bn, eps, d_x);
+  hipStream_t st = (hipStream_t)stream;
+  if (d_next_w && next_dtype == KTX_SEQ_BF16)
+    gated_norm_add_kernel<bf16_t><<<T, 256, (size_t)W * 4, st>>>(W, d_y, ldy, d_ybias, d_ey, d_pair_pos, d_topk_w, top, d_gl, ldg, d_gbias, d_wn,
+                                                                 d_bn, eps, d_x, d_next_w, d_next_b, next_eps, (bf16_t*)d_next_out);
+  else
+    gated_norm_add_kernel<float><<<T, 256, (size_t)W * 4, st>>>(W, d_y, ldy, d_ybias, d_ey, d_pair_pos, d_topk_w, top, d_gl, ldg, d_gbias, d_wn,
+                                                                d_bn, eps, d_x, d_next_w, d_next_b, next_eps, (float*)d_next_out);
   KTX_HIP(hipGetLastError());
   return 0;
 }
@@ -1132,14 +1158,15 @@ int ktx_delta_forward(const ktx_delta_config* cfg, int B, const int32_t* d_q_ind
   if (B == 0) return 0;
   const unsigned blocks = (unsigned)B * cfg->heads * ((cfg->vdim + 63) / 64);
   hipStream_t st = (hipStream_t)stream;
-  // eight wavefronts per workgroup once a quarter of the rows is more than 8: the per-token step is bound by a wavefront's rows
+  // more wavefronts per workgroup as dim grows: a token's step costs a fixed latency plus a term per row a wavefront owns (at dim 128
+  // sixteen wavefronts of 8 rows are no faster than eight of 16: the wider barrier and reduction eat the gain)
 #define KTX_DL_GO(DPW, NW) delta_fwd_kernel<DPW, NW><<<blocks, NW * 64, 0, st>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_qkv, d_gb, d_S, d_o)
   const int D = cfg->dim;
   if (D <= 16) KTX_DL_GO(4, 4);
   else if (D <= 32) KTX_DL_GO(8, 4);
   else if (D <= 64) KTX_DL_GO(8, 8);
   else if (D <= 128) KTX_DL_GO(16, 8);
-  else KTX_DL_GO(32, 8);
+  else KTX_DL_GO(16, 16);
 #undef KTX_DL_GO
   KTX_HIP(hipGetLastError());
   return 0;

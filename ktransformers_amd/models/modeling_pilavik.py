@@ -161,22 +161,32 @@ class PilavikLayer(nn.Module):
         if self.mlp is not None:
             self.norm2, self.norm2b, self.rg2 = PilavikNorm(W, eps), PilavikNorm(W, eps), PilavikGate(W)
 
-    def forward(self, x, batch, cache, cache_idx):
+    def forward(self, x, batch, cache, cache_idx, h=None, next_norm=None):
         """x <- x + norm1b(mix(h) * sigmoid(rg1 h)), h = norm1(x); then the same with the feed-forward.  x is the fp32 residual and is
         updated in place.  The gate's product rides in the sublayer's input GEMM; gate, post-norm, output bias, the mixture's weighted
-        sum and the residual add are the post-norm's one launch."""
-        h = self.norm1(x)
+        sum, the residual add AND the pre-norm of whatever follows are the post-norm's one launch: `h` is norm1(x) when the caller
+        already has it, `next_norm` the pre-norm of the next layer run; returns (x, next_norm(x) or None)."""
+        fused = hasattr(self.norm1b, "gated_add") and hasattr(self.norm1, "weight_f32")
+
+        def after(post, nxt, **kw):
+            if nxt is not None and fused:
+                return post.gated_add(x, next_norm=nxt, **kw)[1]
+            post.gated_add(x, **kw)
+            return nxt(x) if nxt is not None else None
+
+        if h is None:
+            h = self.norm1(x)
         y, gl = self.mix(h, batch, cache, cache_idx, rider=self.rg1)
-        self.norm1b.gated_add(x, y=y, gate_logits=gl, gate_bias=self.rg1.bias_f32)
+        h = after(self.norm1b, self.norm2 if self.mlp is not None else next_norm, y=y, gate_logits=gl, gate_bias=self.rg1.bias_f32)
         if self.mlp is not None:
-            h = self.norm2(x)
             if getattr(self.mlp, "RETURNS_EXPERT_ROWS", False):
                 y, gl, rows, pair_pos, topk_w = self.mlp(h, rider=self.rg2)
-                self.norm2b.gated_add(x, y=y, gate_logits=gl, gate_bias=self.rg2.bias_f32, expert_rows=rows, pair_pos=pair_pos, topk_w=topk_w)
+                h = after(self.norm2b, next_norm, y=y, gate_logits=gl, gate_bias=self.rg2.bias_f32, expert_rows=rows, pair_pos=pair_pos,
+                          topk_w=topk_w)
             else:
                 y, gl = self.mlp(h, rider=self.rg2)
-                self.norm2b.gated_add(x, y=y, ybias=self.mlp.down_bias, gate_logits=gl, gate_bias=self.rg2.bias_f32)
-        return x
+                h = after(self.norm2b, next_norm, y=y, ybias=self.mlp.down_bias, gate_logits=gl, gate_bias=self.rg2.bias_f32)
+        return x, h
 
 
 class _Final(nn.Module):
@@ -219,11 +229,13 @@ class PilavikForCausalLM(nn.Module):
                 logits_rows = torch.tensor([batch.T - 1], dtype=torch.int32, device=cache.device)
         x = self.embed(input_ids, batch.positions)
         x0 = x.clone() if self.config.loop is not None and self.config.loop["times"] > 1 else None
-        trail = []
-        for run, (i, opens_pass) in enumerate(self.config.runs):
+        trail, h, runs = [], None, self.config.runs
+        for run, (i, opens_pass) in enumerate(runs):
             if opens_pass is not None:
                 self.loop(x, x0, opens_pass)
-            x = getattr(self, f"l{i}")(x, batch, cache, run)
+            # the pre-norm of the next run is computed by this run's last launch, unless something is added to x in between
+            follows = getattr(self, f"l{runs[run + 1][0]}").norm1 if run + 1 < len(runs) and runs[run + 1][1] is None else None
+            x, h = getattr(self, f"l{i}")(x, batch, cache, run, h=h, next_norm=follows)
             if return_layers:
                 trail.append(x.clone())
         h = self.final.norm(x, rows=logits_rows, out_dtype=self.config.compute_dtype)

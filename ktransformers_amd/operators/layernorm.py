@@ -68,7 +68,8 @@ class KLayerNormBias(BaseInjectedModule):
       type (`ktx_layer_norm`);
     * BEHIND a sublayer (`gated_add(x, y, ...)`): x += norm(z), z = the sublayer's result — optionally plus its output bias and plus the
       weighted rows of a mixture of experts — times sigmoid(gate logits + gate bias) when a gate is given; one launch
-      (`ktx_gated_norm_add`).
+      (`ktx_gated_norm_add`).  With `next_norm=` (another KLayerNormBias: the pre-norm of the sublayer that follows) the same launch
+      also writes that norm of the updated rows, and the call returns (x, h).
 
     Checkpoint tensors: the module's key (weight) and `<key>.b` (bias, optional)."""
 
@@ -94,7 +95,9 @@ class KLayerNormBias(BaseInjectedModule):
         from ktransformers_amd._native_hyb import layer_norm
         return layer_norm(x, self.weight_f32, self.bias_f32, self.eps, rows=rows, out_dtype=out_dtype or self.compute_dtype or torch.float32)
 
-    def gated_add(self, x, y=None, ybias=None, gate_logits=None, gate_bias=None, expert_rows=None, pair_pos=None, topk_w=None):
+    def gated_add(self, x, y=None, ybias=None, gate_logits=None, gate_bias=None, expert_rows=None, pair_pos=None, topk_w=None, next_norm=None):
+        import torch
         from ktransformers_amd._native_hyb import gated_norm_add
+        nn_ = None if next_norm is None else (next_norm.weight_f32, next_norm.bias_f32, next_norm.eps, next_norm.compute_dtype or torch.float32)
         return gated_norm_add(x, self.weight_f32, self.bias_f32, self.eps, y=y, ybias=ybias, gate_logits=gate_logits, gate_bias=gate_bias,
-                              expert_rows=expert_rows, pair_pos=pair_pos, topk_w=topk_w)
+                              expert_rows=expert_rows, pair_pos=pair_pos, topk_w=topk_w, next_norm=nn_)

@@ -199,7 +199,7 @@ def dense_mlp(ff=48):
     return {"kind": "dense", "ff": ff}
 
 
-def moe_mlp(experts=6, top=2, ff=24, scale=1.5, shared_ff=24):
+def moe_mlp(experts=6, top=2, ff=24, scale=1.25, shared_ff=24):
     return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top, "scale": scale},
             "shared": {"ff": shared_ff} if shared_ff else None}
 
